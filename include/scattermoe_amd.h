@@ -1,0 +1,124 @@
+/*
+ * scattermoe_amd — C ABI of the MI355X (gfx950) ScatterMoE hot path.
+ *
+ * Every entry point is `extern "C"`, takes plain pointers / sizes / element strides, launches
+ * asynchronously on the HIP stream it is given, allocates nothing, frees nothing and keeps no
+ * pointer after it returns.  Device pointers are passed as `void*`; strides are in ELEMENTS of the
+ * tensor's dtype.  Return value: 0 = launched, >0 = the hipError_t of a failed launch,
+ * <0 = argument error (SMOE_ERR_*); `smoe_last_error()` gives the text for the calling thread.
+ *
+ * The reference (shawntan/scattermoe) has no FFI: its Python wrappers launch Triton kernels.  Each
+ * function below names the reference wrapper + kernel it replaces.
+ *
+ * Notation: T tokens, k = top-k, L = T*k rows in expert-sorted order, E experts.
+ *   eid[L]  sorted_expert_idxs      (int64, ascending)
+ *   idx[L]  sorted_scattered_idxs   (int64, permutation of 0..L-1; token = idx / k)
+ *   off[E]  expert_offsets          (int64, inclusive prefix sum of per-expert row counts)
+ */
+#ifndef SCATTERMOE_AMD_H
+#define SCATTERMOE_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SMOE_ABI_VERSION 1
+
+/* element types of floating-point tensors */
+enum { SMOE_F32 = 0, SMOE_BF16 = 1, SMOE_F16 = 2 };
+/* element types of the unsorted expert-index tensor handed to smoe_route */
+enum { SMOE_I64 = 0, SMOE_I32 = 1, SMOE_I16 = 2, SMOE_U8 = 3 };
+
+/* argument errors */
+enum {
+  SMOE_ERR_NULL = -1,      /* a required pointer is NULL */
+  SMOE_ERR_SHAPE = -2,     /* negative / inconsistent sizes */
+  SMOE_ERR_DTYPE = -3,     /* unknown dtype enum */
+  SMOE_ERR_WORKSPACE = -4, /* workspace too small */
+  SMOE_ERR_RANGE = -5      /* size beyond what the kernels index with (int32 rows, E limit) */
+};
+
+/* ABI version of the loaded library (== SMOE_ABI_VERSION it was built with). */
+int smoe_version(void);
+
+/* Text of the last error raised on the calling thread ("" if none). Never NULL. */
+const char* smoe_last_error(void);
+
+/*
+ * Routing prep: stable counting sort of the flattened expert ids + inclusive per-expert offsets.
+ * Replaces scattermoe/parallel_experts.py:14-21 (flatten_sort_count: torch.sort + bincount + cumsum,
+ * with the custom op scattermoe::bincount :6-12).  Tie order is the stable one (ascending flat slot
+ * inside an expert segment), i.e. torch.sort(flat, stable=True).
+ *   expert_idxs  L unsorted ids in [0,E), contiguous, dtype `idx_dtype` (SMOE_I64 ...)
+ *   eid_out/idx_out  L int64 each;  off_out  E int64
+ *   workspace    device scratch of at least smoe_route_workspace_bytes(L,E) bytes (may be NULL iff that is 0)
+ * Ids outside [0,E) are undefined behaviour in the reference; here such rows are dropped from the
+ * histogram and the outputs are unspecified (no out-of-bounds access happens).
+ */
+size_t smoe_route_workspace_bytes(int64_t L, int E);
+int smoe_route(const void* expert_idxs, int idx_dtype, int64_t L, int E,
+               int64_t* eid_out, int64_t* idx_out, int64_t* off_out,
+               void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Inclusive expert offsets from an already sorted id vector (off[e] = #{n : eid[n] <= e}).
+ * The reference's scatter2scatter (scattermoe/kernels/ops.py:120-137) receives only eid/idx and
+ * re-derives expert boundaries per 128-row block (ops.py:85-91); this library schedules
+ * expert-aligned tiles from `off`, so callers that hold no offsets build them with this call.
+ */
+int smoe_offsets_from_sorted(const int64_t* eid, int64_t L, int E, int64_t* off_out, void* stream);
+
+/*
+ * Fused gather -> grouped GEMM (+bias) -> scatter.
+ * Replaces scattermoe/kernels/ops.py:120-183 (scatter2scatter / op scattermoe::scatter2scatter)
+ * and its Triton kernel ops.py:11-42, 50-118.
+ *   for n in [0,L): e = eid[n]; src = x_grouped ? n : idx[n] / fan_out; dst = y_grouped ? n : idx[n]
+ *                   Y[dst, :] = X[src, :] @ W[e] (+ b[e]);  fp32 accumulation, stored in `dtype`
+ *   X (L/fan_out or L rows, K)  strides sxm,sxk     W (E,K,N) strides swe,swk,swn (any layout)
+ *   b (E,N) or NULL  strides sbe,sbn                Y (L,N) strides sym,syn
+ * `off` (E int64) is required.  X, W, b, Y share `dtype`.
+ */
+int smoe_scatter2scatter(const void* X, int64_t sxm, int64_t sxk,
+                         const void* W, int64_t swe, int64_t swk, int64_t swn,
+                         const void* b, int64_t sbe, int64_t sbn,
+                         void* Y, int64_t sym, int64_t syn,
+                         const int64_t* eid, const int64_t* idx, const int64_t* off,
+                         int64_t L, int64_t K, int64_t N, int E, int fan_out,
+                         int x_grouped, int y_grouped, int dtype, void* stream);
+
+/*
+ * Row gather into expert-sorted order with optional per-row coefficient.
+ * Replaces scattermoe/kernels/ops.py:377-410 (group / op scattermoe::group), kernel ops.py:413-457.
+ *   Y[n, :] = A[idx[n] / fan_out, :] * (coeff ? coeff[idx[n]] : 1)      n in [0,L)
+ *   A (L/fan_out, K) strides sam,sak;  coeff (L) contiguous or NULL;  Y (L,K) strides sym,syk
+ */
+int smoe_group(const void* A, int64_t sam, int64_t sak, const void* coeff,
+               void* Y, int64_t sym, int64_t syk, const int64_t* idx,
+               int64_t L, int64_t K, int fan_out, int dtype, void* stream);
+
+/*
+ * Per-expert weight / bias gradient over contiguous expert-sorted row ranges.
+ * Replaces scattermoe/kernels/ops.py:191-239 (group_bwd_W / op scattermoe::groupXtY), kernels
+ * ops.py:242-318, 321-366.
+ *   rows(e) = [e ? off[e-1] : 0, off[e])
+ *   DW[e] (K x N) = sum_{r in rows(e)} X[r,:]^T DY[r,:]       Db[e] (N) = sum_{r in rows(e)} DY[r,:]
+ * Unlike the reference, which relies on a torch.zeros pre-fill (ops.py:192-195) for experts without
+ * rows (guard at ops.py:279), every element of DW / Db is written here (zeros for empty experts),
+ * so the caller may pass uninitialised memory.  fp32 accumulation, fixed summation order.
+ *   DY (L,N) strides sdym,sdyn;  X (L,K) strides sxm,sxk;  DW (E,K,N) strides sdwe,sdwk,sdwn;
+ *   Db (E,N) strides sdbe,sdbn or NULL.
+ */
+int smoe_groupXtY(const void* DY, int64_t sdym, int64_t sdyn,
+                  const void* X, int64_t sxm, int64_t sxk,
+                  void* DW, int64_t sdwe, int64_t sdwk, int64_t sdwn,
+                  void* Db, int64_t sdbe, int64_t sdbn,
+                  const int64_t* off, int64_t L, int64_t K, int64_t N, int E,
+                  int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SCATTERMOE_AMD_H */

@@ -1,0 +1,62 @@
+"""Compile the HIP sources under csrc/ into libscattermoe_amd.so (gfx950 only).
+
+hipcc cross-compiles without a GPU, so this runs on any machine with ROCm.  The library is
+placed inside the package directory and loaded from there by `_C`.
+"""
+import os
+import shutil
+import subprocess
+from concurrent.futures import ThreadPoolExecutor
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(PKG_DIR, "csrc")
+OBJ_DIR = os.path.join(CSRC, "build")
+LIB_PATH = os.path.join(PKG_DIR, "libscattermoe_amd.so")
+
+SOURCES = ["capi.hip", "route.hip", "group.hip", "s2s_generic.hip", "xty_generic.hip", "gemm_mfma.hip"]
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+    # keep the compiler from forming packed fp32 VALU ops
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _hipcc():
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found: the scattermoe_amd kernels need the ROCm toolchain to build")
+    return exe
+
+
+def _run(cmd):
+    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if p.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), p.stdout))
+    return p.stdout
+
+
+def build(verbose=False, jobs=None):
+    """Compile every source and link the shared library; always recompiles."""
+    hipcc = _hipcc()
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    objs = [os.path.join(OBJ_DIR, s.replace(".hip", ".o")) for s in SOURCES]
+
+    def one(pair):
+        src, obj = pair
+        out = _run([hipcc] + HIPCC_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj])
+        if verbose and out.strip():
+            print(out)
+
+    jobs = jobs or min(len(SOURCES), max(1, (os.cpu_count() or 2)), 16)
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        list(ex.map(one, zip(SOURCES, objs)))
+    tmp = LIB_PATH + ".tmp"
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp] + objs)
+    os.replace(tmp, LIB_PATH)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

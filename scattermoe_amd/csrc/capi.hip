@@ -1,0 +1,109 @@
+// extern "C" entry points: argument validation, dispatch between the MFMA and the layout-agnostic
+// kernels.  Nothing here allocates; every launch goes to the caller's stream.
+#include "common.hpp"
+#include <cstdarg>
+#include <cstdio>
+
+namespace smoe {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+int launch_status(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess) return 0;
+  set_error("%s: launch failed: %s", what, hipGetErrorString(e));
+  return (int)e;
+}
+
+static bool dtype_ok(int d) { return d == SMOE_F32 || d == SMOE_BF16 || d == SMOE_F16; }
+
+}  // namespace smoe
+
+using namespace smoe;
+
+extern "C" {
+
+int smoe_version(void) { return SMOE_ABI_VERSION; }
+
+const char* smoe_last_error(void) { return g_err; }
+
+size_t smoe_route_workspace_bytes(int64_t L, int E) {
+  if (L < 0 || E <= 0) return 0;
+  return route_workspace_bytes(L, E);
+}
+
+int smoe_route(const void* expert_idxs, int idx_dtype, int64_t L, int E, int64_t* eid_out,
+               int64_t* idx_out, int64_t* off_out, void* workspace, size_t workspace_bytes, void* stream) {
+  g_err[0] = 0;
+  if (L < 0 || E <= 0) { set_error("smoe_route: bad sizes L=%lld E=%d", (long long)L, E); return SMOE_ERR_SHAPE; }
+  if (L > 0x7fffffffLL) { set_error("smoe_route: L=%lld does not fit int32 row indexing", (long long)L); return SMOE_ERR_RANGE; }
+  if (!off_out || (L > 0 && (!expert_idxs || !eid_out || !idx_out))) { set_error("smoe_route: NULL pointer"); return SMOE_ERR_NULL; }
+  const size_t need = route_workspace_bytes(L, E);
+  if (need > 0 && (!workspace || workspace_bytes < need)) {
+    set_error("smoe_route: workspace of %zu bytes needed, %zu given", need, workspace ? workspace_bytes : (size_t)0);
+    return SMOE_ERR_WORKSPACE;
+  }
+  return launch_route(expert_idxs, idx_dtype, L, E, eid_out, idx_out, off_out, workspace, (hipStream_t)stream);
+}
+
+int smoe_offsets_from_sorted(const int64_t* eid, int64_t L, int E, int64_t* off_out, void* stream) {
+  g_err[0] = 0;
+  if (L < 0 || E <= 0) { set_error("smoe_offsets_from_sorted: bad sizes"); return SMOE_ERR_SHAPE; }
+  if (!off_out || (L > 0 && !eid)) { set_error("smoe_offsets_from_sorted: NULL pointer"); return SMOE_ERR_NULL; }
+  return launch_offsets_from_sorted(eid, L, E, off_out, (hipStream_t)stream);
+}
+
+int smoe_scatter2scatter(const void* X, int64_t sxm, int64_t sxk, const void* W, int64_t swe, int64_t swk,
+                         int64_t swn, const void* b, int64_t sbe, int64_t sbn, void* Y, int64_t sym,
+                         int64_t syn, const int64_t* eid, const int64_t* idx, const int64_t* off, int64_t L,
+                         int64_t K, int64_t N, int E, int fan_out, int x_grouped, int y_grouped, int dtype,
+                         void* stream) {
+  g_err[0] = 0;
+  if (!dtype_ok(dtype)) { set_error("smoe_scatter2scatter: unknown dtype %d", dtype); return SMOE_ERR_DTYPE; }
+  if (L < 0 || K < 0 || N < 0 || E <= 0 || fan_out <= 0) { set_error("smoe_scatter2scatter: bad sizes"); return SMOE_ERR_SHAPE; }
+  if (L > 0x7fffffffLL || K > 0x7fffffffLL || N > 0x7fffffffLL) { set_error("smoe_scatter2scatter: size beyond int32"); return SMOE_ERR_RANGE; }
+  if (L == 0 || N == 0) return 0;
+  if (!X || !W || !Y || !idx || !off) { set_error("smoe_scatter2scatter: NULL pointer"); return SMOE_ERR_NULL; }
+  (void)eid;  // expert boundaries come from `off`; kept in the signature for parity with the reference call
+  S2SArgs a{X, sxm, sxk, W, swe, swk, swn, b, sbe, sbn, Y, sym, syn, eid, idx, off,
+            (int)L, (int)K, (int)N, E, fan_out, x_grouped, y_grouped};
+  int rc = 0;
+  if (try_s2s_mfma(a, dtype, (hipStream_t)stream, rc)) return rc;
+  return launch_s2s_generic(a, dtype, (hipStream_t)stream);
+}
+
+int smoe_group(const void* A, int64_t sam, int64_t sak, const void* coeff, void* Y, int64_t sym, int64_t syk,
+               const int64_t* idx, int64_t L, int64_t K, int fan_out, int dtype, void* stream) {
+  g_err[0] = 0;
+  if (!dtype_ok(dtype)) { set_error("smoe_group: unknown dtype %d", dtype); return SMOE_ERR_DTYPE; }
+  if (L < 0 || K < 0 || fan_out <= 0) { set_error("smoe_group: bad sizes"); return SMOE_ERR_SHAPE; }
+  if (L > 0x7fffffffLL || K > 0x7fffffffLL) { set_error("smoe_group: size beyond int32"); return SMOE_ERR_RANGE; }
+  if (L == 0 || K == 0) return 0;
+  if (!A || !Y || !idx) { set_error("smoe_group: NULL pointer"); return SMOE_ERR_NULL; }
+  GroupArgs a{A, sam, sak, coeff, Y, sym, syk, idx, (int)L, (int)K, fan_out};
+  return launch_group(a, dtype, (hipStream_t)stream);
+}
+
+int smoe_groupXtY(const void* DY, int64_t sdym, int64_t sdyn, const void* X, int64_t sxm, int64_t sxk,
+                  void* DW, int64_t sdwe, int64_t sdwk, int64_t sdwn, void* Db, int64_t sdbe, int64_t sdbn,
+                  const int64_t* off, int64_t L, int64_t K, int64_t N, int E, int dtype, void* stream) {
+  g_err[0] = 0;
+  if (!dtype_ok(dtype)) { set_error("smoe_groupXtY: unknown dtype %d", dtype); return SMOE_ERR_DTYPE; }
+  if (L < 0 || K < 0 || N < 0 || E <= 0) { set_error("smoe_groupXtY: bad sizes"); return SMOE_ERR_SHAPE; }
+  if (L > 0x7fffffffLL || K > 0x7fffffffLL || N > 0x7fffffffLL) { set_error("smoe_groupXtY: size beyond int32"); return SMOE_ERR_RANGE; }
+  if (K == 0 || N == 0) return 0;
+  if (!DW || !off || (L > 0 && (!DY || !X))) { set_error("smoe_groupXtY: NULL pointer"); return SMOE_ERR_NULL; }
+  XtYArgs a{DY, sdym, sdyn, X, sxm, sxk, DW, sdwe, sdwk, sdwn, Db, sdbe, sdbn, off, (int)L, (int)K, (int)N, E};
+  int rc = 0;
+  if (try_xty_mfma(a, dtype, (hipStream_t)stream, rc)) return rc;
+  return launch_xty_generic(a, dtype, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,114 @@
+// Shared device/host helpers for the gfx950 ScatterMoE kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+#include "../../include/scattermoe_amd.h"
+
+namespace smoe {
+
+typedef __bf16 bf16_t;
+typedef _Float16 f16_t;
+
+// ---- error text, one slot per host thread -------------------------------------------------------
+void set_error(const char* fmt, ...);
+int launch_status(const char* what);  // hipGetLastError() -> return code (+ error text)
+
+// ---- element conversion --------------------------------------------------------------------------
+template <typename T> __device__ __forceinline__ float to_f32(T v) { return (float)v; }
+template <typename T> __device__ __forceinline__ T from_f32(float v) { return (T)v; }
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
+
+// ---- expert-aligned tile lookup -------------------------------------------------------------------
+// Rows are expert-sorted; expert e owns rows [off[e-1], off[e]).  Tiles of height BM never straddle
+// two experts: expert e contributes ceil(count_e / BM) tiles and tiles are numbered expert-major.
+// Every wave of the block runs this redundantly and gets the same (uniform) answer.
+// Returns false when `t` is past the last tile (the grid is sized by the host-known upper bound
+// floor(L/BM) + E, so surplus blocks simply exit).
+template <int BM>
+__device__ __forceinline__ bool find_tile(const int64_t* __restrict__ off, int E, int t,
+                                          int& expert, int& row_start, int& rows) {
+  const int lane = lane_id();
+  int tiles_before = 0;
+  for (int e0 = 0; e0 < E; e0 += 64) {
+    const int e = e0 + lane;
+    int lo = 0, hi = 0;
+    if (e < E) {
+      hi = (int)off[e];
+      lo = e ? (int)off[e - 1] : 0;
+    }
+    const int nt = (hi - lo + BM - 1) / BM;
+    int incl = nt;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      int v = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += v;
+    }
+    const int cum = tiles_before + incl;
+    const unsigned long long hit = __ballot(cum > t);
+    if (hit) {
+      const int src = __ffsll((long long)hit) - 1;
+      const int lo_s = __shfl(lo, src, 64), hi_s = __shfl(hi, src, 64);
+      const int first = __shfl(cum - nt, src, 64);
+      expert = e0 + src;
+      row_start = lo_s + (t - first) * BM;
+      rows = min(BM, hi_s - row_start);
+      return true;
+    }
+    tiles_before += __shfl(incl, 63, 64);
+  }
+  return false;
+}
+
+static inline int64_t cdiv64(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Upper bound on the number of expert-aligned tiles of height bm over L rows and E experts.
+static inline int64_t max_tiles(int64_t L, int E, int bm) {
+  int64_t a = L / bm + E;        // sum ceil(c_e/bm) <= floor(L/bm) + E
+  int64_t b = L;                 // and never more than one tile per row
+  int64_t r = a < b ? a : b;
+  return r < 1 ? 1 : r;
+}
+
+// ---- kernel launchers implemented in the individual .hip files ---------------------------------------
+struct S2SArgs {
+  const void* X; int64_t sxm, sxk;
+  const void* W; int64_t swe, swk, swn;
+  const void* b; int64_t sbe, sbn;
+  void* Y; int64_t sym, syn;
+  const int64_t* eid; const int64_t* idx; const int64_t* off;
+  int L, K, N, E, fan_out;
+  int x_grouped, y_grouped;
+};
+
+struct XtYArgs {
+  const void* DY; int64_t sdym, sdyn;
+  const void* X; int64_t sxm, sxk;
+  void* DW; int64_t sdwe, sdwk, sdwn;
+  void* Db; int64_t sdbe, sdbn;
+  const int64_t* off;
+  int L, K, N, E;
+};
+
+struct GroupArgs {
+  const void* A; int64_t sam, sak;
+  const void* coeff;
+  void* Y; int64_t sym, syk;
+  const int64_t* idx;
+  int L, K, fan_out;
+};
+
+int launch_s2s_generic(const S2SArgs& a, int dtype, hipStream_t st);
+int launch_xty_generic(const XtYArgs& a, int dtype, hipStream_t st);
+int launch_group(const GroupArgs& a, int dtype, hipStream_t st);
+// MFMA paths return 1 if they took the call, 0 if the shape/layout is not theirs, <0 / >1 never.
+bool try_s2s_mfma(const S2SArgs& a, int dtype, hipStream_t st, int& rc);
+bool try_xty_mfma(const XtYArgs& a, int dtype, hipStream_t st, int& rc);
+
+int launch_route(const void* expert_idxs, int idx_dtype, int64_t L, int E, int64_t* eid_out,
+                 int64_t* idx_out, int64_t* off_out, void* ws, hipStream_t st);
+size_t route_workspace_bytes(int64_t L, int E);
+int launch_offsets_from_sorted(const int64_t* eid, int64_t L, int E, int64_t* off, hipStream_t st);
+
+}  // namespace smoe

@@ -1,0 +1,73 @@
+// Row gather into expert-sorted order, optionally scaled by a per-row coefficient.
+// Counterpart of group (scattermoe/kernels/ops.py:377-410) and its kernel _group (ops.py:413-457):
+//   Y[n, :] = A[idx[n] / fan_out, :] * coeff[idx[n]]
+// Pure HBM traffic: one wave moves one row in 16-byte pieces when rows are contiguous and aligned,
+// element-wise otherwise.  The product is formed in fp32 and rounded once to the tensor dtype.
+#include "common.hpp"
+
+namespace smoe {
+
+static constexpr int kGroupThreads = 256;
+static constexpr int kGroupRowsPerBlock = kGroupThreads / 64;
+
+template <typename T> struct Vec16 { static constexpr int n = 16 / sizeof(T); T v[16 / sizeof(T)]; };
+
+template <typename T, bool VEC>
+__global__ __launch_bounds__(kGroupThreads) void group_kernel(GroupArgs a) {
+  const T* __restrict__ A = (const T*)a.A;
+  const T* __restrict__ coeff = (const T*)a.coeff;
+  T* __restrict__ Y = (T*)a.Y;
+  const int lane = lane_id();
+  const int wave = threadIdx.x >> 6;
+  for (int64_t n = (int64_t)blockIdx.x * kGroupRowsPerBlock + wave; n < a.L;
+       n += (int64_t)gridDim.x * kGroupRowsPerBlock) {
+    const int64_t i = a.idx[n];
+    const int64_t src = i / a.fan_out;
+    const float c = coeff ? to_f32(coeff[i]) : 1.0f;
+    const T* __restrict__ s = A + src * a.sam;
+    T* __restrict__ d = Y + n * a.sym;
+    if (VEC) {
+      typedef Vec16<T> V;
+      const int nv = a.K / V::n;
+      for (int j = lane; j < nv; j += 64) {
+        V x = *(const V*)(s + (int64_t)j * V::n);
+        if (coeff) {
+#pragma unroll
+          for (int q = 0; q < V::n; ++q) x.v[q] = from_f32<T>(to_f32(x.v[q]) * c);
+        }
+        *(V*)(d + (int64_t)j * V::n) = x;
+      }
+    } else {
+      for (int j = lane; j < a.K; j += 64) {
+        const float x = to_f32(s[(int64_t)j * a.sak]);
+        d[(int64_t)j * a.syk] = coeff ? from_f32<T>(x * c) : from_f32<T>(x);
+      }
+    }
+  }
+}
+
+template <typename T>
+static int launch_group_t(const GroupArgs& a, hipStream_t st) {
+  if (a.L == 0 || a.K == 0) return 0;
+  constexpr int vn = 16 / sizeof(T);
+  const bool vec = a.sak == 1 && a.syk == 1 && a.K % vn == 0 && a.sam % vn == 0 && a.sym % vn == 0 &&
+                   ((uintptr_t)a.A % 16 == 0) && ((uintptr_t)a.Y % 16 == 0);
+  int64_t blocks = cdiv64(a.L, kGroupRowsPerBlock);
+  if (blocks > 256 * 64) blocks = 256 * 64;   // grid-stride beyond 64 blocks per CU
+  if (vec)
+    hipLaunchKernelGGL((group_kernel<T, true>), dim3((unsigned)blocks), dim3(kGroupThreads), 0, st, a);
+  else
+    hipLaunchKernelGGL((group_kernel<T, false>), dim3((unsigned)blocks), dim3(kGroupThreads), 0, st, a);
+  return launch_status("group_kernel");
+}
+
+int launch_group(const GroupArgs& a, int dtype, hipStream_t st) {
+  switch (dtype) {
+    case SMOE_F32: return launch_group_t<float>(a, st);
+    case SMOE_BF16: return launch_group_t<bf16_t>(a, st);
+    case SMOE_F16: return launch_group_t<f16_t>(a, st);
+    default: set_error("smoe_group: unknown dtype %d", dtype); return SMOE_ERR_DTYPE;
+  }
+}
+
+}  // namespace smoe

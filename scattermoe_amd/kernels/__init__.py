@@ -1,0 +1,3 @@
+from . import ops
+
+__all__ = ["ops"]

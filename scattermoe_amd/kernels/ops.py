@@ -1,0 +1,241 @@
+"""Host half of the expert kernels: output allocation, shape checks, and the hand-off to the C ABI.
+
+Mirrors the wrapper layer of the reference, scattermoe/kernels/ops.py — `scatter2scatter` (:120-137),
+`group_bwd_W` (:191-199), `group` (:377-386) and the four `torch.library` ops (:140, :202, :389 and
+parallel_experts.py:6) — with the Triton launches replaced by calls into libscattermoe_amd.so.
+
+All device work goes through `_backend`, an object with `route / offsets / s2s / group / xty` methods.
+The only backend shipped is `HipBackend` (the C ABI); it refuses CPU tensors.
+"""
+from typing import Optional
+
+import torch
+
+from .. import _C
+
+# Kept so that code written against the reference keeps working.  Tile heights are picked inside the
+# library per launch, and gfx950 has no TF32 mode: fp32 inputs are always multiplied in full fp32.
+BLOCK_M = 128
+ALLOW_TF32 = True
+
+
+class HipBackend:
+    """Launches the gfx950 kernels on the current torch stream of the tensors' device."""
+
+    name = "hip"
+
+    @staticmethod
+    def route(flat_ids, num_experts, eid, idx, off):
+        _C.require_gpu(flat_ids, "flatten_sort_count")
+        lib = _C.load()
+        L = flat_ids.numel()
+        need = lib.smoe_route_workspace_bytes(L, num_experts)
+        ws = torch.empty(need, dtype=torch.uint8, device=flat_ids.device) if need else None
+        with torch.cuda.device(flat_ids.device):
+            rc = lib.smoe_route(_C.ptr(flat_ids), _C.index_code(flat_ids.dtype), L, num_experts,
+                                _C.ptr(eid), _C.ptr(idx), _C.ptr(off), _C.ptr(ws), need,
+                                _C.stream_ptr(flat_ids.device))
+        _C.check(rc, "smoe_route")
+
+    @staticmethod
+    def offsets(eid, num_experts, off):
+        _C.require_gpu(eid, "expert offsets")
+        lib = _C.load()
+        with torch.cuda.device(eid.device):
+            rc = lib.smoe_offsets_from_sorted(_C.ptr(eid), eid.numel(), num_experts, _C.ptr(off),
+                                              _C.stream_ptr(eid.device))
+        _C.check(rc, "smoe_offsets_from_sorted")
+
+    @staticmethod
+    def s2s(X, W, b, Y, eid, idx, off, k, x_grouped, y_grouped):
+        _C.require_gpu(X, "scatter2scatter")
+        lib = _C.load()
+        sbe, sbn = (b.stride(0), b.stride(1)) if b is not None else (0, 0)
+        with torch.cuda.device(X.device):
+            rc = lib.smoe_scatter2scatter(
+                _C.ptr(X), X.stride(0), X.stride(1),
+                _C.ptr(W), W.stride(0), W.stride(1), W.stride(2),
+                _C.ptr(b), sbe, sbn,
+                _C.ptr(Y), Y.stride(0), Y.stride(1),
+                _C.ptr(eid), _C.ptr(idx), _C.ptr(off),
+                eid.numel(), X.size(1), Y.size(1), W.size(0), k,
+                int(bool(x_grouped)), int(bool(y_grouped)), _C.float_code(X.dtype),
+                _C.stream_ptr(X.device))
+        _C.check(rc, "smoe_scatter2scatter")
+
+    @staticmethod
+    def group(A, coeff, Y, idx, fan_out):
+        _C.require_gpu(A, "group")
+        lib = _C.load()
+        with torch.cuda.device(A.device):
+            rc = lib.smoe_group(_C.ptr(A), A.stride(0), A.stride(1), _C.ptr(coeff),
+                                _C.ptr(Y), Y.stride(0), Y.stride(1), _C.ptr(idx),
+                                idx.numel(), A.size(1), fan_out, _C.float_code(A.dtype),
+                                _C.stream_ptr(A.device))
+        _C.check(rc, "smoe_group")
+
+    @staticmethod
+    def xty(DY, X, DW, Db, off, E):
+        _C.require_gpu(DY, "group_bwd_W")
+        lib = _C.load()
+        sdbe, sdbn = (Db.stride(0), Db.stride(1)) if Db is not None else (0, 0)
+        with torch.cuda.device(DY.device):
+            rc = lib.smoe_groupXtY(
+                _C.ptr(DY), DY.stride(0), DY.stride(1),
+                _C.ptr(X), X.stride(0), X.stride(1),
+                _C.ptr(DW), DW.stride(0), DW.stride(1), DW.stride(2),
+                _C.ptr(Db), sdbe, sdbn,
+                _C.ptr(off), DY.size(0), X.size(1), DY.size(1), E, _C.float_code(DY.dtype),
+                _C.stream_ptr(DY.device))
+        _C.check(rc, "smoe_groupXtY")
+
+
+_backend = HipBackend()
+
+
+def _same_dtype(what, ref, *others):
+    for t in others:
+        if t is not None and t.dtype != ref.dtype:
+            raise TypeError("%s: dtype mismatch (%s vs %s)" % (what, ref.dtype, t.dtype))
+
+
+def _as_i64(t):
+    return t if t.dtype == torch.int64 else t.to(torch.int64)
+
+
+# ------------------------------------------------------------------------------------------------
+# routing prep
+# ------------------------------------------------------------------------------------------------
+def route(expert_idxs: torch.Tensor, num_experts: int):
+    """Stable sort of the flattened expert ids; returns (sorted ids, source slots, inclusive offsets)."""
+    flat = expert_idxs.reshape(-1)
+    if not flat.is_contiguous():
+        flat = flat.contiguous()
+    if flat.dtype not in (torch.int64, torch.int32, torch.int16, torch.uint8):
+        flat = flat.to(torch.int64)
+    L = flat.numel()
+    eid = torch.empty(L, dtype=torch.int64, device=flat.device)
+    idx = torch.empty(L, dtype=torch.int64, device=flat.device)
+    off = torch.empty(num_experts, dtype=torch.int64, device=flat.device)
+    _backend.route(flat, num_experts, eid, idx, off)
+    return eid, idx, off
+
+
+def offsets_from_sorted(sorted_expert_idxs: torch.Tensor, num_experts: int):
+    off = torch.empty(num_experts, dtype=torch.int64, device=sorted_expert_idxs.device)
+    _backend.offsets(_as_i64(sorted_expert_idxs).contiguous(), num_experts, off)
+    return off
+
+
+# ------------------------------------------------------------------------------------------------
+# scatter2scatter
+# ------------------------------------------------------------------------------------------------
+def scatter2scatter(X, W, sorted_expert_idxs, sorted_scattered_idxs, k,
+                    b=None, x_grouped=False, y_grouped=False, out=None, expert_offsets=None):
+    """Y[dst(n)] = X[src(n)] @ W[eid[n]] (+ b[eid[n]]) over the L expert-sorted rows.
+
+    Same contract as the reference wrapper (ops.py:120-137).  `expert_offsets` is an optional extra:
+    callers that already hold the inclusive offsets pass them and save one small launch.
+    """
+    L = sorted_expert_idxs.size(0)
+    assert sorted_scattered_idxs.size(0) == L
+    assert L == X.size(0) * k
+    assert W.dim() == 3 and W.size(1) == X.size(1)
+    N = W.size(-1)
+    if out is None:
+        out = torch.empty((L, N), device=X.device, dtype=X.dtype)
+    else:
+        assert out.size(0) == L and out.size(1) == N
+    if torch.compiler.is_compiling():
+        scatter2scatter_compileable(out, W, X, k, sorted_expert_idxs, sorted_scattered_idxs,
+                                    b, x_grouped, y_grouped)
+    else:
+        _s2s_launch(out, W, X, k, sorted_expert_idxs, sorted_scattered_idxs, b,
+                    x_grouped, y_grouped, expert_offsets)
+    return out
+
+
+def _s2s_launch(out, W, X, k, eid, idx, b, x_grouped, y_grouped, off):
+    _same_dtype("scatter2scatter", X, W, b, out)
+    eid, idx = _as_i64(eid).contiguous(), _as_i64(idx).contiguous()
+    if off is None:
+        off = offsets_from_sorted(eid, W.size(0))
+    else:
+        off = _as_i64(off).contiguous()
+        assert off.numel() == W.size(0)
+    _backend.s2s(X, W, b, out, eid, idx, off, k, x_grouped, y_grouped)
+
+
+@torch.library.custom_op("scattermoe::scatter2scatter", mutates_args={"output"})
+def scatter2scatter_compileable(
+        output: torch.Tensor, W: torch.Tensor, X: torch.Tensor, k: int,
+        sorted_expert_idxs: torch.Tensor, sorted_scattered_idxs: torch.Tensor,
+        b: Optional[torch.Tensor], x_grouped: bool, y_grouped: bool) -> None:
+    _s2s_launch(output, W, X, k, sorted_expert_idxs, sorted_scattered_idxs, b, x_grouped, y_grouped, None)
+
+
+# ------------------------------------------------------------------------------------------------
+# groupXtY
+# ------------------------------------------------------------------------------------------------
+def group_bwd_W(DY, X, expert_offsets, E, has_bias=False):
+    """Per-expert dW / db over expert-grouped rows (reference ops.py:191-199).
+
+    The returned DW is an (E, K, N) view of a contiguous (E, N, K) buffer, so that after autograd undoes
+    the `weight.permute(0, 2, 1)` of ParallelExperts the parameter gradient is contiguous.  The kernel
+    writes every element (zeros for experts without rows), hence `empty` rather than `zeros`.
+    """
+    N, K = DY.size(-1), X.size(-1)
+    DWt = torch.empty((E, N, K), device=DY.device, dtype=DY.dtype)
+    DW = DWt.permute(0, 2, 1)
+    Db = torch.empty((E, N), device=DY.device, dtype=DY.dtype) if has_bias else None
+    if torch.compiler.is_compiling():
+        groupXtY_compileable(E, DW, Db, DY, X, expert_offsets)
+    else:
+        _xty_launch(E, DW, Db, DY, X, expert_offsets)
+    return DW, Db
+
+
+def _xty_launch(E, DW, Db, DY, X, expert_offsets):
+    assert DY.size(0) == X.size(0)
+    assert expert_offsets.numel() == E
+    _same_dtype("group_bwd_W", DY, X, DW, Db)
+    _backend.xty(DY, X, DW, Db, _as_i64(expert_offsets).contiguous(), E)
+
+
+@torch.library.custom_op("scattermoe::groupXtY", mutates_args={"DW", "Db"})
+def groupXtY_compileable(E: int, DW: torch.Tensor, Db: Optional[torch.Tensor],
+                         DY: torch.Tensor, X: torch.Tensor, expert_offsets: torch.Tensor) -> None:
+    _xty_launch(E, DW, Db, DY, X, expert_offsets)
+
+
+# ------------------------------------------------------------------------------------------------
+# group
+# ------------------------------------------------------------------------------------------------
+def group(A, sorted_expert_idxs, coeff=None, fan_out=1, out=None):
+    """Y[n] = A[idx[n] // fan_out] * coeff[idx[n]]  (reference ops.py:377-386).
+
+    As in the reference the second argument is, despite its name, the sorted *scattered* index vector.
+    """
+    N, K = sorted_expert_idxs.size(0), A.size(1)
+    assert A.size(0) * fan_out == N
+    Y = out if out is not None else torch.empty((N, K), dtype=A.dtype, device=A.device)
+    if torch.compiler.is_compiling():
+        group_compileable(A, K, N, Y, coeff, coeff is not None, fan_out, sorted_expert_idxs)
+    else:
+        _group_launch(A, Y, coeff, fan_out, sorted_expert_idxs)
+    return Y
+
+
+def _group_launch(A, Y, coeff, fan_out, idx):
+    assert Y.size(0) == idx.size(0) and Y.size(1) == A.size(1)
+    _same_dtype("group", A, Y)
+    if coeff is not None:
+        assert coeff.numel() == idx.size(0)
+        coeff = coeff.reshape(-1).to(A.dtype).contiguous()
+    _backend.group(A, coeff, Y, _as_i64(idx).contiguous(), fan_out)
+
+
+@torch.library.custom_op("scattermoe::group", mutates_args={"Y"})
+def group_compileable(A: torch.Tensor, K: int, N: int, Y: torch.Tensor, coeff: Optional[torch.Tensor],
+                      has_coeff: bool, fan_out: int, sorted_expert_idxs: torch.Tensor) -> None:
+    _group_launch(A, Y, coeff if has_coeff else None, fan_out, sorted_expert_idxs)

@@ -1,0 +1,177 @@
+"""GPU parity of each C-ABI entry point against the CPU oracle on identical seeded inputs.
+Integer outputs bit-exact; floating point: fp32 rel 1e-4, bf16/fp16 rel 2e-2 / abs 1e-2."""
+import itertools
+
+import pytest
+import torch
+
+import oracle
+from scattermoe_amd.kernels import ops
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+TOL = {torch.float32: dict(rtol=1e-4, atol=1e-5), torch.bfloat16: dict(rtol=2e-2, atol=1e-2),
+       torch.float16: dict(rtol=2e-2, atol=1e-2)}
+
+
+def _close(got, want, dtype, scale=1.0):
+    t = TOL[dtype]
+    got, want = got.float().cpu(), want.float().cpu()
+    err = (got - want).abs()
+    bound = t["atol"] * scale + t["rtol"] * want.abs()
+    assert bool((err <= bound).all()), "max err %g (bound %g)" % (err.max(), bound.flatten()[err.argmax()])
+
+
+def _experts(T, E, k, seed, skew=False):
+    g = torch.Generator().manual_seed(seed)
+    logits = torch.randn(T, E, generator=g)
+    if skew:
+        logits = logits - 1.8 * torch.log(torch.arange(1, E + 1, dtype=torch.float32))
+    return torch.topk(logits, k).indices
+
+
+# ---------------------------------------------------------------------------------------------------
+# routing: bit-exact
+# ---------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("T,E,k", [(1, 8, 2), (3, 1, 1), (256, 8, 2), (512, 8, 4), (2048, 8, 2), (2049, 8, 2),
+                                   (8192, 32, 4), (32768, 128, 8), (16384, 8, 2), (5000, 300, 3), (70000, 64, 1)])
+@pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
+def test_route_bit_exact(T, E, k, dtype):
+    experts = _experts(T, E, k, seed=T + E, skew=(E >= 32)).to(dtype)
+    eid, idx, off = ops.route(experts.to(DEV), E)
+    r_eid, r_idx, r_off = oracle.route_ref(experts, E)
+    assert eid.dtype == idx.dtype == off.dtype == torch.int64
+    assert torch.equal(eid.cpu(), r_eid) and torch.equal(idx.cpu(), r_idx) and torch.equal(off.cpu(), r_off)
+    s_eid, s_idx = torch.sort(experts.flatten().long(), stable=True)
+    assert torch.equal(eid.cpu(), s_eid) and torch.equal(idx.cpu(), s_idx)
+
+
+def test_route_edge_cases():
+    flat = torch.full((5000,), 3, dtype=torch.int64)                      # one expert takes everything
+    eid, idx, off = ops.route(flat.to(DEV), 6)
+    assert torch.equal(idx.cpu(), torch.arange(5000)) and off.tolist() == [0, 0, 0, 5000, 5000, 5000]
+    eid, idx, off = ops.route(torch.empty(0, 2, dtype=torch.int64, device=DEV), 4)   # no rows
+    assert eid.numel() == 0 and off.tolist() == [0, 0, 0, 0]
+    u8 = torch.tensor([[7, 0], [0, 7]], dtype=torch.uint8)
+    eid, idx, off = ops.route(u8.to(DEV), 8)
+    assert eid.tolist() == [0, 0, 7, 7] and idx.tolist() == [1, 2, 0, 3] and off.tolist() == [2] * 7 + [4]
+    a = ops.route(_experts(4096, 16, 4, 1).to(DEV), 16)
+    b = ops.route(_experts(4096, 16, 4, 1).to(DEV), 16)
+    assert all(torch.equal(x, y) for x, y in zip(a, b))                   # run-to-run identical
+
+
+def test_offsets_from_sorted():
+    for E, L in [(8, 1000), (40, 77), (5, 0), (128, 9000)]:
+        eid = torch.sort(torch.randint(0, E, (L,))).values
+        if L:
+            eid[eid == 1] = 0                                             # an empty expert
+            eid = torch.sort(eid).values
+        off = ops.offsets_from_sorted(eid.to(DEV), E)
+        assert torch.equal(off.cpu(), torch.bincount(eid, minlength=E).cumsum(0))
+
+
+# ---------------------------------------------------------------------------------------------------
+# scatter2scatter
+# ---------------------------------------------------------------------------------------------------
+S2S_SHAPES = [  # T, E, k, K, N
+    (1, 8, 2, 128, 128), (77, 8, 3, 100, 133), (256, 8, 2, 128, 256), (300, 8, 4, 600, 150),
+    (512, 16, 2, 64, 72), (1024, 8, 2, 256, 512), (2048, 8, 2, 512, 384),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("w_layout", ["k_contig", "n_contig"])
+@pytest.mark.parametrize("T,E,k,K,N", S2S_SHAPES)
+def test_scatter2scatter_forward_layer(T, E, k, K, N, w_layout, dtype):
+    g = torch.Generator().manual_seed(K * 7 + N)
+    experts = _experts(T, E, k, seed=T)
+    eid, idx, off = oracle.route_ref(experts, E)
+    X = torch.randn(T, K, generator=g).to(dtype)
+    Wp = (torch.randn(E, N, K, generator=g) * 0.1).to(dtype)
+    W = Wp.permute(0, 2, 1) if w_layout == "k_contig" else Wp.permute(0, 2, 1).contiguous()
+    b = torch.randn(E, N, generator=g).to(dtype)
+    want = oracle.scatter2scatter_ref(X.float(), W.float(), eid, idx, k, b.float(), False, True)
+    Wd = Wp.to(DEV).permute(0, 2, 1) if w_layout == "k_contig" else W.to(DEV)
+    got = ops.scatter2scatter(X.to(DEV), Wd, eid.to(DEV), idx.to(DEV), k, b=b.to(DEV), y_grouped=True,
+                              expert_offsets=off.to(DEV))
+    assert got.dtype == dtype
+    _close(got, want, dtype, scale=K ** 0.5 * 0.1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("x_grouped,y_grouped", list(itertools.product([False, True], repeat=2)))
+def test_scatter2scatter_grouping_modes(x_grouped, y_grouped, dtype):
+    T, E, k, K, N = 700, 8, 2, 256, 192
+    g = torch.Generator().manual_seed(12)
+    experts = _experts(T, E, k, seed=3, skew=True)
+    experts[experts == 5] = 4                                             # expert 5 has no rows
+    eid, idx, off = oracle.route_ref(experts, E)
+    fan = 1 if x_grouped else k
+    X = torch.randn(T * k // fan, K, generator=g).to(dtype)
+    W = (torch.randn(E, K, N, generator=g) * 0.1).to(dtype)
+    want = oracle.scatter2scatter_ref(X.float(), W.float(), eid, idx, fan, None, x_grouped, y_grouped)
+    # offsets omitted on purpose: the wrapper derives them from the sorted ids like the reference signature
+    got = ops.scatter2scatter(X.to(DEV), W.to(DEV), eid.to(DEV), idx.to(DEV), fan,
+                              x_grouped=x_grouped, y_grouped=y_grouped)
+    _close(got, want, dtype, scale=K ** 0.5 * 0.1)
+    out = torch.full((T * k, N), float("nan"), dtype=dtype, device=DEV)
+    ret = ops.scatter2scatter(X.to(DEV), W.to(DEV), eid.to(DEV), idx.to(DEV), fan, x_grouped=x_grouped,
+                              y_grouped=y_grouped, out=out)
+    assert ret.data_ptr() == out.data_ptr() and torch.equal(ret, got)     # out= is filled completely, deterministically
+
+
+def test_scatter2scatter_e1_is_plain_gemm():
+    T, K, N = 1000, 384, 320
+    g = torch.Generator().manual_seed(0)
+    X = torch.randn(T, K, generator=g)
+    W = torch.randn(1, K, N, generator=g) * 0.05
+    eid, idx, off = oracle.route_ref(torch.zeros(T, 1, dtype=torch.long), 1)
+    got = ops.scatter2scatter(X.to(DEV), W.to(DEV), eid.to(DEV), idx.to(DEV), 1)
+    _close(got, X @ W[0], torch.float32, scale=K ** 0.5 * 0.05)
+
+
+# ---------------------------------------------------------------------------------------------------
+# group
+# ---------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,k,K", [(1, 2, 128), (333, 3, 100), (1024, 2, 4096), (257, 4, 72)])
+@pytest.mark.parametrize("with_coeff", [False, True])
+def test_group_bit_exact(T, k, K, with_coeff, dtype):
+    g = torch.Generator().manual_seed(T + K)
+    experts = _experts(T, 8, k, seed=K)
+    _, idx, _ = oracle.route_ref(experts, 8)
+    A = torch.randn(T, K, generator=g).to(dtype)
+    coeff = torch.rand(T, k, generator=g).to(dtype) if with_coeff else None
+    want = oracle.group_ref(A, idx, None if coeff is None else coeff.flatten(), fan_out=k)
+    got = ops.group(A.to(DEV), idx.to(DEV), coeff=None if coeff is None else coeff.flatten().to(DEV), fan_out=k)
+    assert torch.equal(got.cpu(), want)          # a copy with one correctly rounded product: bit-exact
+    sub = torch.randn(T, K + 8, generator=g).to(dtype)                    # strided source rows
+    got2 = ops.group(sub.to(DEV)[:, 3:K + 3], idx.to(DEV), fan_out=k)
+    assert torch.equal(got2.cpu(), oracle.group_ref(sub[:, 3:K + 3], idx, None, k))
+
+
+# ---------------------------------------------------------------------------------------------------
+# groupXtY
+# ---------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,E,k,K,N", [(1, 8, 2, 128, 128), (77, 8, 3, 100, 133), (512, 8, 2, 256, 128),
+                                       (1500, 16, 2, 192, 320), (2048, 4, 2, 512, 256)])
+def test_group_bwd_W(T, E, k, K, N, dtype):
+    g = torch.Generator().manual_seed(N + 3 * K)
+    experts = _experts(T, E, k, seed=T + 1, skew=True)
+    eid, idx, off = oracle.route_ref(experts, E)
+    L = T * k
+    X = torch.randn(L, K, generator=g).to(dtype)
+    DY = (torch.randn(L, N, generator=g) * 0.1).to(dtype)
+    DW_ref, Db_ref = oracle.group_bwd_W_ref(DY.float(), X.float(), off, E, has_bias=True)
+    DW, Db = ops.group_bwd_W(DY.to(DEV), X.to(DEV), off.to(DEV), E, has_bias=True)
+    assert DW.shape == (E, K, N) and DW.permute(0, 2, 1).is_contiguous() and Db.shape == (E, N)
+    rows = torch.diff(off, prepend=torch.zeros(1, dtype=torch.long)).max().item()
+    _close(DW, DW_ref, dtype, scale=rows ** 0.5 * 0.1)
+    _close(Db, Db_ref, dtype, scale=rows ** 0.5 * 0.1)
+    empty = (torch.diff(off, prepend=torch.zeros(1, dtype=torch.long)) == 0).nonzero().flatten()
+    for e in empty.tolist():
+        assert not DW[e].any() and not Db[e].any()                        # written as exact zeros
+    DW2, _ = ops.group_bwd_W(DY.to(DEV), X.to(DEV), off.to(DEV), E, has_bias=False)
+    assert torch.equal(DW2, DW)                                           # fixed summation order

@@ -1,0 +1,259 @@
+"""Pins the CPU oracle against facts that do not depend on its own formulas: brute-force loops over
+Python floats, closed forms, finite-difference gradients and Hugging Face's independent expert loops.
+The reference keeps no golden vectors (tests/test_mlp.py draws unseeded inputs), so these are the pins."""
+import itertools
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+
+
+def _rand_routing(T, E, k, seed):
+    g = torch.Generator().manual_seed(seed)
+    probs = torch.softmax(torch.randn(T, E, generator=g), -1)
+    p, experts = torch.topk(probs, k)
+    return p, experts
+
+
+# ---------------------------------------------------------------------------------------------------
+# routing
+# ---------------------------------------------------------------------------------------------------
+def _route_bruteforce(flat, E):
+    pairs = []
+    for e in range(E):                      # expert-major, original position ascending = stable order
+        for pos, v in enumerate(flat):
+            if v == e:
+                pairs.append((e, pos))
+    counts = [sum(1 for v in flat if v == e) for e in range(E)]
+    off, run = [], 0
+    for c in counts:
+        run += c
+        off.append(run)
+    return [p[0] for p in pairs], [p[1] for p in pairs], off
+
+
+@pytest.mark.parametrize("T,E,k", [(1, 8, 2), (5, 3, 2), (17, 8, 3), (64, 4, 4), (9, 1, 1), (33, 16, 2)])
+def test_route_bruteforce(T, E, k):
+    _, experts = _rand_routing(T, E, k, seed=T * 131 + E)
+    eid, idx, off = oracle.route_ref(experts, E)
+    b_eid, b_idx, b_off = _route_bruteforce(experts.flatten().tolist(), E)
+    assert eid.tolist() == b_eid and idx.tolist() == b_idx and off.tolist() == b_off
+    assert eid.dtype == idx.dtype == off.dtype == torch.int64
+
+
+def test_route_invariants_and_torch_stable_sort():
+    g = torch.Generator().manual_seed(3)
+    flat = torch.randint(0, 7, (4099,), generator=g)
+    flat[flat == 5] = 4                      # expert 5 stays empty
+    eid, idx, off = oracle.route_ref(flat, 7)
+    s_eid, s_idx = torch.sort(flat, stable=True)
+    assert torch.equal(eid, s_eid) and torch.equal(idx, s_idx)
+    assert torch.equal(off, torch.bincount(flat, minlength=7).cumsum(0))
+    assert torch.equal(torch.sort(idx).values, torch.arange(flat.numel()))        # permutation
+    assert torch.equal(flat[idx], eid) and bool((eid[1:] >= eid[:-1]).all())
+    same = eid[1:] == eid[:-1]
+    assert bool((idx[1:][same] > idx[:-1][same]).all())                          # stable inside a segment
+    assert off[-1] == flat.numel() and off[5] == off[4]
+
+
+def test_route_special_cases():
+    assert [t.tolist() for t in oracle.route_ref(torch.tensor([[2]]), 4)] == [[2], [0], [0, 0, 1, 1]]
+    eid, idx, off = oracle.route_ref(torch.full((6, 2), 3), 5)                   # everything to one expert
+    assert eid.tolist() == [3] * 12 and idx.tolist() == list(range(12)) and off.tolist() == [0, 0, 0, 12, 12]
+    eid, idx, off = oracle.route_ref(torch.tensor([1, 0, 1, 0], dtype=torch.int32), 2)  # flat, int32 input
+    assert eid.tolist() == [0, 0, 1, 1] and idx.tolist() == [1, 3, 0, 2] and off.tolist() == [2, 4]
+
+
+# ---------------------------------------------------------------------------------------------------
+# kernel models vs brute force
+# ---------------------------------------------------------------------------------------------------
+def _s2s_bruteforce(X, W, eid, idx, k, b, x_grouped, y_grouped):
+    L, K, N = len(eid), len(X[0]), len(W[0][0])
+    Y = [[0.0] * N for _ in range(L)]
+    for n in range(L):
+        e = eid[n]
+        src = n if x_grouped else idx[n] // k
+        dst = n if y_grouped else idx[n]
+        for j in range(N):
+            s = math.fsum(X[src][c] * W[e][c][j] for c in range(K))
+            Y[dst][j] = s + (b[e][j] if b is not None else 0.0)
+    return Y
+
+
+@pytest.mark.parametrize("x_grouped,y_grouped", list(itertools.product([False, True], repeat=2)))
+@pytest.mark.parametrize("bias", [False, True])
+def test_scatter2scatter_bruteforce(x_grouped, y_grouped, bias):
+    T, E, k, K, N = 7, 3, 2, 5, 4
+    g = torch.Generator().manual_seed(11)
+    _, experts = _rand_routing(T, E, k, seed=5)
+    eid, idx, _ = oracle.route_ref(experts, E)
+    fan = 1 if x_grouped else k
+    X = torch.randn(T * k // fan, K, generator=g, dtype=torch.float64)
+    W = torch.randn(E, K, N, generator=g, dtype=torch.float64)
+    b = torch.randn(E, N, generator=g, dtype=torch.float64) if bias else None
+    got = oracle.scatter2scatter_ref(X, W, eid, idx, fan, b, x_grouped, y_grouped, acc=torch.float64)
+    want = _s2s_bruteforce(X.tolist(), W.tolist(), eid.tolist(), idx.tolist(), fan,
+                           None if b is None else b.tolist(), x_grouped, y_grouped)
+    assert torch.allclose(got, torch.tensor(want, dtype=torch.float64), atol=1e-12, rtol=0)
+
+
+def test_scatter2scatter_closed_forms():
+    g = torch.Generator().manual_seed(2)
+    T, k, K, N = 6, 2, 4, 4
+    # E = 1: a plain linear layer applied to every (token, slot) row
+    X = torch.randn(T, K, generator=g)
+    W = torch.randn(1, K, N, generator=g)
+    eid, idx, _ = oracle.route_ref(torch.zeros(T, k, dtype=torch.long), 1)
+    Y = oracle.scatter2scatter_ref(X, W, eid, idx, k)
+    assert torch.allclose(Y, F.linear(X, W[0].T).repeat_interleave(k, 0), atol=1e-6)
+    # identity weights copy the routed token into its slot row; a strided (transposed) W view is honoured
+    _, experts = _rand_routing(T, 3, k, seed=9)
+    eid, idx, _ = oracle.route_ref(experts, 3)
+    eye = torch.eye(K).expand(3, K, K)
+    assert torch.equal(oracle.scatter2scatter_ref(X, eye, eid, idx, k), X.repeat_interleave(k, 0))
+    Wt = torch.randn(3, N, K, generator=g)
+    a = oracle.scatter2scatter_ref(X, Wt.permute(0, 2, 1), eid, idx, k)
+    b = oracle.scatter2scatter_ref(X, Wt.permute(0, 2, 1).contiguous(), eid, idx, k)
+    assert torch.allclose(a, b, atol=1e-6)
+    # one-hot rows pick out row c of the routed expert's matrix
+    Xh = torch.zeros(T, K); Xh[:, 2] = 1.0
+    Yh = oracle.scatter2scatter_ref(Xh, Wt.permute(0, 2, 1), eid, idx, k)
+    assert torch.equal(Yh, Wt[experts.flatten(), :, 2])
+
+
+def test_group_and_group_bwd_W_bruteforce():
+    g = torch.Generator().manual_seed(4)
+    T, E, k, K, N = 9, 4, 2, 3, 5
+    p, experts = _rand_routing(T, E, k, seed=8)
+    experts[experts == 2] = 1                                   # expert 2 empty
+    eid, idx, off = oracle.route_ref(experts, E)
+    A = torch.randn(T, K, generator=g, dtype=torch.float64)
+    coeff = p.double()
+    got = oracle.group_ref(A, idx, coeff.flatten(), fan_out=k)
+    for n in range(T * k):
+        i = int(idx[n])
+        assert torch.allclose(got[n], A[i // k] * coeff.flatten()[i], atol=1e-15)
+    assert torch.equal(oracle.group_ref(A, idx, None, fan_out=k), A[idx // k])
+    Xg = torch.randn(T * k, K, generator=g, dtype=torch.float64)
+    DY = torch.randn(T * k, N, generator=g, dtype=torch.float64)
+    DW, Db = oracle.group_bwd_W_ref(DY, Xg, off, E, has_bias=True, acc=torch.float64)
+    for e in range(E):
+        rows = [n for n in range(T * k) if int(eid[n]) == e]
+        for c in range(K):
+            for j in range(N):
+                want = math.fsum(float(Xg[r, c]) * float(DY[r, j]) for r in rows)
+                assert abs(float(DW[e, c, j]) - want) < 1e-12
+        for j in range(N):
+            assert abs(float(Db[e, j]) - math.fsum(float(DY[r, j]) for r in rows)) < 1e-12
+    assert not DW[2].any() and not Db[2].any()
+
+
+# ---------------------------------------------------------------------------------------------------
+# the naive MoE MLP
+# ---------------------------------------------------------------------------------------------------
+def _mlp_bruteforce(x, p, experts, W1, W2, b1, b2, act):
+    T, k = len(experts), len(experts[0])
+    out = []
+    for t in range(T):
+        y = [0.0] * len(W2[0])
+        for j in range(k):
+            e = experts[t][j]
+            h = [act(math.fsum(W1[e][r][c] * x[t][c] for c in range(len(x[t]))) + (b1[e][r] if b1 else 0.0))
+                 for r in range(len(W1[e]))]
+            for o in range(len(W2[e])):
+                v = math.fsum(W2[e][o][r] * h[r] for r in range(len(h))) + (b2[e][o] if b2 else 0.0)
+                y[o] += p[t][j] * v
+        out.append(y)
+    return out
+
+
+@pytest.mark.parametrize("bias", [False, True])
+def test_naive_forms_vs_bruteforce(bias):
+    g = torch.Generator().manual_seed(21)
+    T, E, k, d, f = 5, 3, 2, 4, 6
+    p, experts = _rand_routing(T, E, k, seed=1)
+    p = p.double()
+    x = torch.randn(T, d, generator=g, dtype=torch.float64)
+    W1 = torch.randn(E, f, d, generator=g, dtype=torch.float64)
+    W2 = torch.randn(E, d, f, generator=g, dtype=torch.float64)
+    b1 = torch.randn(E, f, generator=g, dtype=torch.float64) if bias else None
+    b2 = torch.randn(E, d, generator=g, dtype=torch.float64) if bias else None
+    want = torch.tensor(_mlp_bruteforce(x.tolist(), p.tolist(), experts.tolist(), W1.tolist(), W2.tolist(),
+                                        b1.tolist() if bias else None, b2.tolist() if bias else None,
+                                        math.tanh), dtype=torch.float64)
+    a = oracle.naive_token_forward(x, p, experts, W1, W2, torch.tanh, b1, b2)
+    b = oracle.naive_expert_forward(x, p, experts, W1, W2, torch.tanh, b1, b2)
+    assert torch.allclose(a, want, atol=1e-12) and torch.allclose(b, want, atol=1e-12)
+
+
+def test_token_form_equals_expert_form_c1_shape():
+    from _inputs import CONFIGS, make_inputs
+    cfg = CONFIGS["c1"]
+    t = make_inputs(cfg)
+    act = torch.nn.GELU()
+    a = oracle.naive_token_forward(t["x"][:64], t["p"][:64], t["experts"][:64], t["W1"], t["W2"], act)
+    b = oracle.naive_expert_forward(t["x"][:64], t["p"][:64], t["experts"][:64], t["W1"], t["W2"], act)
+    assert torch.allclose(a, b, atol=1e-6)
+
+
+def test_glu_split_convention():
+    pre = torch.tensor([[1.0, 2.0, 3.0, 4.0]])
+    # first half linear, second half activated
+    assert torch.allclose(oracle.glu(torch.tanh)(pre), torch.tanh(pre[:, 2:]) * pre[:, :2])
+    pre = torch.tensor([[0.5, 9.0, -8.0, -9.0]])
+    gate, up = torch.tensor([0.5, -8.0]), torch.tensor([7.0, -7.0])          # interleaved + clamped
+    want = (up + 1) * gate * torch.sigmoid(1.702 * gate)
+    assert torch.allclose(oracle.gpt_oss_glu()(pre), want[None])
+
+
+def test_naive_expert_forward_gradcheck():
+    g = torch.Generator().manual_seed(5)
+    T, E, k, d, f = 4, 3, 2, 3, 4
+    p, experts = _rand_routing(T, E, k, seed=2)
+    args = [torch.randn(T, d, generator=g, dtype=torch.float64), p.double(),
+            torch.randn(E, 2 * f, d, generator=g, dtype=torch.float64),
+            torch.randn(E, d, f, generator=g, dtype=torch.float64),
+            torch.randn(E, 2 * f, generator=g, dtype=torch.float64),
+            torch.randn(E, d, generator=g, dtype=torch.float64)]
+    for a in args:
+        a.requires_grad_()
+    fn = lambda x, p_, W1, W2, b1, b2: oracle.naive_expert_forward(
+        x, p_, experts, W1, W2, oracle.glu(F.silu), b1, b2)
+    assert torch.autograd.gradcheck(fn, args, eps=1e-6, atol=1e-5)
+
+
+def test_against_huggingface_expert_loops():
+    """Independent implementations: transformers' MixtralExperts / GptOssExperts forward loops."""
+    mixtral = pytest.importorskip("transformers.models.mixtral.modeling_mixtral")
+    gptoss = pytest.importorskip("transformers.models.gpt_oss.modeling_gpt_oss")
+    from transformers import MixtralConfig, GptOssConfig
+    T, E, k, d, f = 12, 4, 2, 8, 16
+    p, experts = _rand_routing(T, E, k, seed=6)
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(T, d, generator=g)
+
+    m = mixtral.MixtralExperts(MixtralConfig(hidden_size=d, intermediate_size=f, num_local_experts=E,
+                                             num_experts_per_tok=k, hidden_act="silu"))
+    with torch.no_grad():
+        m.gate_up_proj.copy_(torch.randn(E, 2 * f, d, generator=g) * 0.3)
+        m.down_proj.copy_(torch.randn(E, d, f, generator=g) * 0.3)
+        want = m(x, experts, p)
+        # HF: act(first half) * second half; the oracle's GLU: act(second half) * first half
+        gate, up = m.gate_up_proj.chunk(2, dim=1)
+        got = oracle.naive_expert_forward(x, p, experts, torch.cat([up, gate], 1), m.down_proj, oracle.glu(F.silu))
+    assert torch.allclose(got, want, atol=1e-5)
+
+    o = gptoss.GptOssExperts(GptOssConfig(hidden_size=d, intermediate_size=f, num_local_experts=E,
+                                          num_experts_per_tok=k))
+    with torch.no_grad():
+        o.gate_up_proj.copy_(torch.randn(E, d, 2 * f, generator=g) * 0.5)
+        o.gate_up_proj_bias.copy_(torch.randn(E, 2 * f, generator=g))
+        o.down_proj.copy_(torch.randn(E, f, d, generator=g) * 0.5)
+        o.down_proj_bias.copy_(torch.randn(E, d, generator=g))
+        want = o(x, experts, p)
+        got = oracle.naive_expert_forward(x, p, experts, o.gate_up_proj.transpose(1, 2), o.down_proj.transpose(1, 2),
+                                          oracle.gpt_oss_glu(o.alpha, o.limit), o.gate_up_proj_bias, o.down_proj_bias)
+    assert torch.allclose(got, want, atol=1e-5)
