@@ -1,5 +1,496 @@
+// bf16 / fp16 MFMA paths of scatter2scatter and groupXtY for gfx950.
+//
+// One workgroup owns one BM x BN output tile that never straddles two experts and walks the
+// contraction in slices of 64: global -> registers -> LDS (double buffered) -> MFMA 32x32x16.
+// Operands whose contraction axis is contiguous in memory ("direct": gathered X rows, weights stored
+// (N,K)) sit in LDS as [row][64] with a 16-byte XOR swizzle and are read with ds_read_b128; operands
+// whose contraction axis is strided ("transposed": weights stored (K,N), both operands of X^T dY) sit
+// as [64][cols] and are read with ds_read_b64_tr_b16, which hands each lane four consecutive
+// contraction elements of one column.
+//
+// Counterparts in the reference: _scatter2scatter + _compute_expert_block
+// (scattermoe/kernels/ops.py:11-42, 50-118) and _groupXtY + _xty_and_bias (ops.py:242-366).
 #include "common.hpp"
+#include <type_traits>
+
 namespace smoe {
-bool try_s2s_mfma(const S2SArgs&, int, hipStream_t, int&) { return false; }
-bool try_xty_mfma(const XtYArgs&, int, hipStream_t, int&) { return false; }
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+static constexpr int BK = 64;               // contraction slice per stage
+static constexpr int kTrPad = 64;           // bytes of padding per row of a transposed LDS tile
+
+template <typename T> struct Mfma;
+template <> struct Mfma<bf16_t> {
+  static __device__ __forceinline__ f32x16 run(i32x4 a, i32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float sum8(i32x4 a) {
+    const bf16x8 v = __builtin_bit_cast(bf16x8, a);
+    return (((float)v[0] + (float)v[1]) + ((float)v[2] + (float)v[3])) +
+           (((float)v[4] + (float)v[5]) + ((float)v[6] + (float)v[7]));
+  }
+};
+template <> struct Mfma<f16_t> {
+  static __device__ __forceinline__ f32x16 run(i32x4 a, i32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float sum8(i32x4 a) {
+    const f16x8 v = __builtin_bit_cast(f16x8, a);
+    return (((float)v[0] + (float)v[1]) + ((float)v[2] + (float)v[3])) +
+           (((float)v[4] + (float)v[5]) + ((float)v[6] + (float)v[7]));
+  }
+};
+
+typedef __attribute__((address_space(3))) char lds_char;
+
+__device__ __forceinline__ i32x4 lds_read16(const char* p) { return *(const i32x4*)p; }
+__device__ __forceinline__ void lds_write16(char* p, i32x4 v) { *(i32x4*)p = v; }
+__device__ __forceinline__ s16x4 lds_read_tr(const char* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p);
 }
+
+// ---- operand with contiguous contraction axis: LDS tile [EXT][64], 128 B per row, swizzled ----------
+__device__ __forceinline__ int direct_off(int row, int chunk) {
+  const int s = (row & 7) ^ ((row >> 3) & 1);
+  return row * 128 + ((chunk ^ s) << 4);
+}
+
+template <int EXT, int NT>
+struct DirectOp {
+  static constexpr int CHUNKS = EXT * 8;
+  static constexpr int R = (CHUNKS + NT - 1) / NT;
+  static constexpr int LDS_BYTES = EXT * 128;
+  const char* ptr[R];      // row base (bytes) of the row this thread copies in round i
+  // `row_ptr(row)` returns the global byte address of element (row, k = 0) of the tile's row `row`
+  template <typename F>
+  __device__ __forceinline__ void init(F row_ptr) {
+    const int t = threadIdx.x;
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      const int c = t + i * NT;
+      ptr[i] = (c < CHUNKS) ? row_ptr(c >> 3) : nullptr;
+    }
+  }
+  __device__ __forceinline__ void load(i32x4 (&regs)[R], int k0, int kend) const {
+    const int kk = k0 + (threadIdx.x & 7) * 8;
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      i32x4 v = {0, 0, 0, 0};
+      if (ptr[i] != nullptr && kk < kend) v = *(const i32x4*)(ptr[i] + (int64_t)kk * 2);
+      regs[i] = v;
+    }
+  }
+  __device__ __forceinline__ void store(char* tile, const i32x4 (&regs)[R]) const {
+    const int t = threadIdx.x;
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      const int c = t + i * NT;
+      if (c < CHUNKS) lds_write16(tile + direct_off(c >> 3, c & 7), regs[i]);
+    }
+  }
+  // fragment of MFMA operand rows [base, base+32), contraction step ks (16 elements)
+  static __device__ __forceinline__ i32x4 frag(const char* tile, int base, int ks) {
+    const int l = lane_id();
+    return lds_read16(tile + direct_off(base + (l & 31), 2 * ks + (l >> 5)));
+  }
+};
+
+// ---- operand with strided contraction axis: LDS tile [64][EXT] (+pad), read transposed ----------------
+template <int EXT, int NT>
+struct TransOp {
+  static constexpr int CPR = EXT / 8;                  // 16-byte chunks per contraction row
+  static constexpr int CHUNKS = 64 * CPR;
+  static constexpr int R = (CHUNKS + NT - 1) / NT;
+  static constexpr int RS = EXT * 2 + kTrPad;          // LDS row stride, bytes
+  static constexpr int LDS_BYTES = 64 * RS;
+  const char* base;   // global byte address of (contraction 0, column 0 of the tile)
+  int64_t ld;         // bytes between contraction rows
+  int ncols;          // valid columns of this tile (multiple of 8)
+  __device__ __forceinline__ void init(const char* b, int64_t ld_bytes, int valid_cols) {
+    base = b; ld = ld_bytes; ncols = valid_cols;
+  }
+  __device__ __forceinline__ void load(i32x4 (&regs)[R], int k0, int kend) const {
+    const int t = threadIdx.x;
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      const int c = t + i * NT;
+      const int kr = c / CPR, cc = c % CPR;
+      i32x4 v = {0, 0, 0, 0};
+      if (c < CHUNKS && k0 + kr < kend && cc * 8 < ncols)
+        v = *(const i32x4*)(base + (int64_t)(k0 + kr) * ld + cc * 16);
+      regs[i] = v;
+    }
+  }
+  __device__ __forceinline__ void store(char* tile, const i32x4 (&regs)[R]) const {
+    const int t = threadIdx.x;
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      const int c = t + i * NT;
+      if (c < CHUNKS) lds_write16(tile + (c / CPR) * RS + (c % CPR) * 16, regs[i]);
+    }
+  }
+  // Each 16-lane block transposes a 4 (contraction) x 16 (columns) patch: lane r of the block points at
+  // contraction row r/4, columns 4*(r%4)..+3 and receives column r, contraction 0..3.  Blocks 0/1 cover
+  // columns 0-15 / 16-31 of the 32-wide fragment, blocks 2/3 the contraction elements 8..15; a second
+  // read 4 rows further down completes the 8 elements per lane the MFMA expects (k = 8*(lane/32) + 0..7).
+  static __device__ __forceinline__ i32x4 frag(const char* tile, int base, int ks) {
+    const int l = lane_id();
+    const int b = l >> 4, r = l & 15;
+    const int col = base + 16 * (b & 1) + 4 * (r & 3);
+    const int kr = ks * 16 + 8 * (b >> 1) + (r >> 2);
+    const char* p = tile + kr * RS + col * 2;
+    const s16x4 lo = lds_read_tr(p);
+    const s16x4 hi = lds_read_tr(p + 4 * RS);
+    const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(i32x4, v);
+  }
+};
+
+template <int BM_, int BN_, int WM_, int WN_>
+struct Tile {
+  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_;
+  static constexpr int NW = WM * WN, NT = NW * 64;
+  static constexpr int WTM = BM / WM, WTN = BN / WN;
+  static constexpr int FM = WTM / 32, FN = WTN / 32;
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA");
+};
+
+// Main loop shared by both kernels.  acc[i][j] is the 32x32 block (i, j) of this wave's tile.
+// If ROWSUM, rs[i] additionally accumulates, per lane, the sum of the lane's own 8 contraction elements of
+// A-fragment i; adding lanes l and l+32 afterwards gives the sum over the contraction of A row l%32.
+template <typename T, class TL, class AOp, class BOp, bool CAN_ROWSUM>
+__device__ __forceinline__ void mainloop(const AOp& A, const BOp& B, int kbeg, int kend, char* lds, bool rowsum,
+                                         f32x16 (&acc)[TL::FM][TL::FN], float (&rs)[TL::FM]) {
+  constexpr int STAGE = AOp::LDS_BYTES + BOp::LDS_BYTES;
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave / TL::WN, wn = wave % TL::WN;
+  const int nk = (kend - kbeg + BK - 1) / BK;
+  i32x4 ra[AOp::R], rb[BOp::R];
+  if (nk > 0) {
+    A.load(ra, kbeg, kend);
+    B.load(rb, kbeg, kend);
+    A.store(lds, ra);
+    B.store(lds + AOp::LDS_BYTES, rb);
+  }
+  __syncthreads();
+  for (int kt = 0; kt < nk; ++kt) {
+    char* cur = lds + (kt & 1) * STAGE;
+    char* nxt = lds + ((kt + 1) & 1) * STAGE;
+    const bool more = kt + 1 < nk;
+    if (more) {
+      A.load(ra, kbeg + (kt + 1) * BK, kend);
+      B.load(rb, kbeg + (kt + 1) * BK, kend);
+    }
+    const char* ta = cur;
+    const char* tb = cur + AOp::LDS_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      i32x4 fa[TL::FM], fb[TL::FN];
+#pragma unroll
+      for (int i = 0; i < TL::FM; ++i) fa[i] = AOp::frag(ta, wm * TL::WTM + i * 32, ks);
+#pragma unroll
+      for (int j = 0; j < TL::FN; ++j) fb[j] = BOp::frag(tb, wn * TL::WTN + j * 32, ks);
+#pragma unroll
+      for (int i = 0; i < TL::FM; ++i)
+#pragma unroll
+        for (int j = 0; j < TL::FN; ++j) acc[i][j] = Mfma<T>::run(fa[i], fb[j], acc[i][j]);
+      if (CAN_ROWSUM && rowsum) {
+#pragma unroll
+        for (int i = 0; i < TL::FM; ++i) rs[i] += Mfma<T>::sum8(fa[i]);
+      }
+    }
+    if (more) {
+      A.store(nxt, ra);
+      B.store(nxt + AOp::LDS_BYTES, rb);
+    }
+    __syncthreads();
+  }
+}
+
+// Store the wave's accumulators.  dst[m] is the element offset of output row m of the tile (or -1),
+// columns n0 + [0, BN) clipped to ncols; optional bias (already offset to the expert) with stride sb.
+template <typename T, class TL>
+__device__ __forceinline__ void epilogue(const f32x16 (&acc)[TL::FM][TL::FN], T* __restrict__ out,
+                                         const int64_t* dst, int n0, int ncols, int64_t scol,
+                                         const T* __restrict__ bias, int64_t sb) {
+  const int wave = threadIdx.x >> 6, l = lane_id();
+  const int wm = wave / TL::WN, wn = wave % TL::WN;
+#pragma unroll
+  for (int j = 0; j < TL::FN; ++j) {
+    const int n = n0 + wn * TL::WTN + j * 32 + (l & 31);
+    const bool nok = n < ncols;
+    const float bv = (bias != nullptr && nok) ? to_f32(bias[(int64_t)n * sb]) : 0.0f;
+#pragma unroll
+    for (int i = 0; i < TL::FM; ++i) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = wm * TL::WTM + i * 32 + (r >> 2) * 8 + (l >> 5) * 4 + (r & 3);
+        const int64_t d = dst[m];
+        if (nok && d >= 0) out[d + (int64_t)n * scol] = from_f32<T>(acc[i][j][r] + bv);
+      }
+    }
+  }
+}
+
+// XCD-aware tile order.  Workgroup ids are dealt round-robin to the 8 XCDs (private L2 each), so
+// XCD x = id % 8 takes column groups x, x+8, ... (GN adjacent column tiles each) and sweeps all row
+// tiles of a column group before moving on: the B panels of a group stay in that XCD's L2 while the
+// row panels being swept are shared by all XCDs through the memory-side cache.
+struct Raster {
+  int m_tiles, n_tiles, gn;
+  __host__ int64_t grid() const {
+    const int supers = (n_tiles + 8 * gn - 1) / (8 * gn);
+    return (int64_t)8 * gn * m_tiles * supers;
+  }
+  __device__ __forceinline__ bool map(int pid, int& m, int& n) const {
+    const int x = pid & 7, i = pid >> 3;
+    const int nl = i % gn;
+    const int rest = i / gn;
+    m = rest % m_tiles;
+    const int sup = rest / m_tiles;
+    n = (sup * 8 + x) * gn + nl;
+    return n < n_tiles;
+  }
+};
+
+static Raster make_raster(int64_t m_tiles, int n_tiles) {
+  Raster r;
+  r.m_tiles = (int)m_tiles;
+  r.n_tiles = n_tiles;
+  r.gn = 1;
+  for (int g = 4; g >= 2; g >>= 1)
+    if (n_tiles % (8 * g) == 0) { r.gn = g; break; }
+  return r;
+}
+
+// =====================================================================================================
+// scatter2scatter
+// =====================================================================================================
+template <typename T, class TL, bool B_TR>
+__global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast) {
+  typedef DirectOp<TL::BM, TL::NT> AOp;
+  typedef typename std::conditional<B_TR, TransOp<TL::BN, TL::NT>, DirectOp<TL::BN, TL::NT>>::type BOp;
+  constexpr int STAGE = AOp::LDS_BYTES + BOp::LDS_BYTES;
+  __shared__ __attribute__((aligned(16))) char lds[2 * STAGE];
+  __shared__ int64_t sDst[TL::BM];
+  __shared__ int sSrc[TL::BM];
+
+  int m_tile, n_tile;
+  if (!rast.map(blockIdx.x, m_tile, n_tile)) return;
+  int e, row0, rows;
+  if (!find_tile<TL::BM>(a.off, a.E, m_tile, e, row0, rows)) return;
+  const int n0 = n_tile * TL::BN;
+
+  for (int m = threadIdx.x; m < TL::BM; m += TL::NT) {
+    const int mm = m < rows ? m : rows - 1;               // tail rows re-read the last valid row
+    const int64_t n = row0 + mm;
+    int64_t src = n, dst = n;
+    if (!a.x_grouped || !a.y_grouped) {
+      const int64_t i = a.idx[n];
+      if (!a.x_grouped) src = i / a.fan_out;
+      if (!a.y_grouped) dst = i;
+    }
+    sSrc[m] = (int)src;
+    sDst[m] = m < rows ? dst * a.sym : -1;
+  }
+  __syncthreads();
+
+  AOp A;
+  const char* Xb = (const char*)a.X;
+  const int64_t sxm = a.sxm;
+  A.init([&](int row) { return Xb + (int64_t)sSrc[row] * sxm * 2; });
+  BOp B;
+  const char* Wb = (const char*)a.W + (int64_t)e * a.swe * 2;
+  if constexpr (B_TR) {
+    B.init(Wb + (int64_t)n0 * 2, a.swk * 2, a.N - n0);
+  } else {
+    const int64_t swn = a.swn;
+    const int N = a.N;
+    B.init([&](int row) { const int n = n0 + row < N ? n0 + row : N - 1; return Wb + (int64_t)n * swn * 2; });
+  }
+
+  f32x16 acc[TL::FM][TL::FN];
+  float rs[TL::FM];
+#pragma unroll
+  for (int i = 0; i < TL::FM; ++i)
+#pragma unroll
+    for (int j = 0; j < TL::FN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+  mainloop<T, TL, AOp, BOp, false>(A, B, 0, a.K, lds, false, acc, rs);
+
+  const T* bias = a.b ? (const T*)a.b + (int64_t)e * a.sbe : nullptr;
+  epilogue<T, TL>(acc, (T*)a.Y, sDst, n0, a.N, a.syn, bias, a.sbn);
+}
+
+template <typename T, class TL>
+static int launch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
+  const int n_tiles = (a.N + TL::BN - 1) / TL::BN;
+  const Raster r = make_raster(max_tiles(a.L, a.E, TL::BM), n_tiles);
+  const int64_t grid = r.grid();
+  if (grid > 0x7fffffffLL) { set_error("smoe_scatter2scatter: grid too large"); return SMOE_ERR_RANGE; }
+  if (b_tr)
+    hipLaunchKernelGGL((s2s_mfma_kernel<T, TL, true>), dim3((unsigned)grid), dim3(TL::NT), 0, st, a, r);
+  else
+    hipLaunchKernelGGL((s2s_mfma_kernel<T, TL, false>), dim3((unsigned)grid), dim3(TL::NT), 0, st, a, r);
+  return launch_status("s2s_mfma_kernel");
+}
+
+template <typename T>
+static int dispatch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
+  const int64_t avg = a.L / a.E;
+  if (avg >= 192) return launch_s2s<T, Tile<256, 256, 2, 4>>(a, b_tr, st);
+  if (avg >= 96) return launch_s2s<T, Tile<128, 256, 2, 4>>(a, b_tr, st);
+  return launch_s2s<T, Tile<64, 256, 2, 4>>(a, b_tr, st);
+}
+
+static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+bool try_s2s_mfma(const S2SArgs& a, int dtype, hipStream_t st, int& rc) {
+  if (dtype != SMOE_BF16 && dtype != SMOE_F16) return false;
+  if (a.K < 8 || a.K % 8 != 0) return false;
+  if (a.sxk != 1 || a.sxm % 8 != 0 || !aligned16(a.X)) return false;
+  if (a.syn != 1) return false;
+  if (!aligned16(a.W) || a.swe % 8 != 0) return false;
+  bool b_tr;
+  if (a.swk == 1 && a.swn % 8 == 0) b_tr = false;
+  else if (a.swn == 1 && a.swk % 8 == 0 && a.N % 8 == 0) b_tr = true;
+  else return false;
+  rc = dtype == SMOE_BF16 ? dispatch_s2s<bf16_t>(a, b_tr, st) : dispatch_s2s<f16_t>(a, b_tr, st);
+  return true;
+}
+
+// =====================================================================================================
+// groupXtY:  OUT[e] (P x Q, Q contiguous) = sum_r  Pm[r, :]^T  Qm[r, :]   over the expert's rows
+//   DW stored (E,N,K)-contiguous (the ParallelExperts layout):  P = dY (N cols), Q = X  (K cols)
+//   DW stored (E,K,N)-contiguous:                              P = X  (K cols), Q = dY (N cols)
+// Column sums of dY (the bias gradient) ride along: the first column of tiles adds up the dY fragments it
+// already holds in registers.
+// =====================================================================================================
+struct XtYPlan {
+  const void* P; int64_t ldp; int np;     // row-operand source: (L, np), leading dimension ldp elements
+  const void* Q; int64_t ldq; int nq;     // column-operand source
+  void* OUT; int64_t soe, sop;            // output: expert stride, row stride (columns contiguous)
+  void* Db; int64_t sdbe, sdbn;
+  const int64_t* off;
+  int E;
+  int db_from_p;                          // 1: dY is P (row sums of the tile), 0: dY is Q
+};
+
+template <typename T, class TL>
+__global__ __launch_bounds__(TL::NT) void xty_mfma_kernel(XtYPlan a, Raster rast, int p_tiles) {
+  typedef TransOp<TL::BM, TL::NT> AOp;
+  typedef TransOp<TL::BN, TL::NT> BOp;
+  constexpr int STAGE = AOp::LDS_BYTES + BOp::LDS_BYTES;
+  __shared__ __attribute__((aligned(16))) char lds[2 * STAGE];
+  __shared__ int64_t sDst[TL::BM];
+
+  int m_tile, n_tile;
+  if (!rast.map(blockIdx.x, m_tile, n_tile)) return;
+  const int e = m_tile / p_tiles;
+  const int p0 = (m_tile % p_tiles) * TL::BM;
+  const int q0 = n_tile * TL::BN;
+  const int r_lo = e ? (int)a.off[e - 1] : 0;
+  const int r_hi = (int)a.off[e];
+
+  for (int m = threadIdx.x; m < TL::BM; m += TL::NT)
+    sDst[m] = (p0 + m < a.np) ? (int64_t)e * a.soe + (int64_t)(p0 + m) * a.sop : -1;
+  __syncthreads();
+
+  AOp A;
+  A.init((const char*)a.P + ((int64_t)r_lo * a.ldp + p0) * 2, a.ldp * 2, a.np - p0);
+  BOp B;
+  B.init((const char*)a.Q + ((int64_t)r_lo * a.ldq + q0) * 2, a.ldq * 2, a.nq - q0);
+
+  f32x16 acc[TL::FM][TL::FN];
+  float rs[TL::FM];
+#pragma unroll
+  for (int i = 0; i < TL::FM; ++i) {
+    rs[i] = 0.0f;
+#pragma unroll
+    for (int j = 0; j < TL::FN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+  }
+  const bool want_db = a.Db != nullptr && a.db_from_p && n_tile == 0;
+  mainloop<T, TL, AOp, BOp, true>(A, B, 0, r_hi - r_lo, lds, want_db, acc, rs);
+
+  epilogue<T, TL>(acc, (T*)a.OUT, sDst, q0, a.nq, 1, nullptr, 0);
+
+  if (want_db) {
+    // lanes l and l+32 hold the two contraction halves of row l%32; the first wave column writes the sums
+    const int wave = threadIdx.x >> 6, l = lane_id();
+    const int wm = wave / TL::WN, wn = wave % TL::WN;
+#pragma unroll
+    for (int i = 0; i < TL::FM; ++i) {
+      const float tot = rs[i] + __shfl_xor(rs[i], 32, 64);
+      const int p = p0 + wm * TL::WTM + i * 32 + l;
+      if (wn == 0 && l < 32 && p < a.np) ((T*)a.Db)[(int64_t)e * a.sdbe + (int64_t)p * a.sdbn] = from_f32<T>(tot);
+    }
+  }
+}
+
+// Bias gradient when dY is the column operand: plain column sums per expert segment.
+template <typename T>
+__global__ __launch_bounds__(256) void colsum_kernel(const T* __restrict__ DY, int64_t ld, int N,
+                                                    const int64_t* __restrict__ off, T* __restrict__ Db,
+                                                    int64_t sdbe, int64_t sdbn) {
+  const int e = blockIdx.y;
+  const int n = blockIdx.x * 256 + threadIdx.x;
+  if (n >= N) return;
+  const int r_lo = e ? (int)off[e - 1] : 0, r_hi = (int)off[e];
+  float s = 0.0f;
+  for (int r = r_lo; r < r_hi; ++r) s += to_f32(DY[(int64_t)r * ld + n]);
+  Db[(int64_t)e * sdbe + (int64_t)n * sdbn] = from_f32<T>(s);
+}
+
+template <typename T>
+static int launch_xty(const XtYArgs& a, hipStream_t st) {
+  typedef Tile<256, 256, 2, 4> TL;
+  XtYPlan p;
+  const bool k_contig = a.sdwk == 1;     // output rows = N index
+  if (k_contig) {
+    p.P = a.DY; p.ldp = a.sdym; p.np = a.N;
+    p.Q = a.X; p.ldq = a.sxm; p.nq = a.K;
+    p.sop = a.sdwn;
+  } else {
+    p.P = a.X; p.ldp = a.sxm; p.np = a.K;
+    p.Q = a.DY; p.ldq = a.sdym; p.nq = a.N;
+    p.sop = a.sdwk;
+  }
+  p.OUT = a.DW; p.soe = a.sdwe;
+  p.Db = a.Db; p.sdbe = a.sdbe; p.sdbn = a.sdbn;
+  p.off = a.off; p.E = a.E;
+  p.db_from_p = k_contig ? 1 : 0;
+  const int p_tiles = (p.np + TL::BM - 1) / TL::BM;
+  const int q_tiles = (p.nq + TL::BN - 1) / TL::BN;
+  const Raster r = make_raster((int64_t)a.E * p_tiles, q_tiles);
+  const int64_t grid = r.grid();
+  if (grid > 0x7fffffffLL) { set_error("smoe_groupXtY: grid too large"); return SMOE_ERR_RANGE; }
+  hipLaunchKernelGGL((xty_mfma_kernel<T, TL>), dim3((unsigned)grid), dim3(TL::NT), 0, st, p, r, p_tiles);
+  int rc = launch_status("xty_mfma_kernel");
+  if (rc == 0 && a.Db != nullptr && !k_contig) {
+    hipLaunchKernelGGL(colsum_kernel<T>, dim3((a.N + 255) / 256, a.E), dim3(256), 0, st, (const T*)a.DY,
+                       a.sdym, a.N, a.off, (T*)a.Db, a.sdbe, a.sdbn);
+    rc = launch_status("colsum_kernel");
+  }
+  return rc;
+}
+
+bool try_xty_mfma(const XtYArgs& a, int dtype, hipStream_t st, int& rc) {
+  if (dtype != SMOE_BF16 && dtype != SMOE_F16) return false;
+  if (a.K % 8 != 0 || a.N % 8 != 0) return false;
+  if (a.sdyn != 1 || a.sxk != 1 || a.sdym % 8 != 0 || a.sxm % 8 != 0) return false;
+  if (!aligned16(a.DY) || !aligned16(a.X)) return false;
+  if (a.sdwk != 1 && a.sdwn != 1) return false;
+  rc = dtype == SMOE_BF16 ? launch_xty<bf16_t>(a, st) : launch_xty<f16_t>(a, st);
+  return true;
+}
+
+}  // namespace smoe

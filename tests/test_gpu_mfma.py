@@ -1,0 +1,122 @@
+"""bf16 / fp16 MFMA paths: shapes that exercise every tile class, contraction and column tails, both
+weight layouts, scatter/gather modes, empty and tiny experts.  Oracle: CPU fp32 on the same rounded
+inputs; tolerance rel 2e-2 / abs 1e-2 (scaled by the magnitude a dot product of that length reaches)."""
+import itertools
+
+import pytest
+import torch
+
+import oracle
+from scattermoe_amd.kernels import ops
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _close(got, want, scale):
+    got, want = got.float().cpu(), want.float().cpu()
+    err = (got - want).abs()
+    bound = 1e-2 * scale + 2e-2 * want.abs()
+    assert bool((err <= bound).all()), "max err %g at bound %g" % (err.max(), bound.flatten()[err.argmax()])
+
+
+def _routing(T, E, k, seed, skew=0.0, empty=()):
+    g = torch.Generator().manual_seed(seed)
+    logits = torch.randn(T, E, generator=g)
+    if skew:
+        logits = logits - skew * torch.log(torch.arange(1, E + 1, dtype=torch.float32))
+    for e in empty:
+        logits[:, e] = -1e9
+    experts = torch.topk(logits, k).indices
+    return experts, oracle.route_ref(experts, E)
+
+
+# T, E, k, K, N  — rows/expert select the 256-, 128- and 64-row tile classes
+SHAPES = [
+    (4096, 8, 2, 512, 768),      # 1024 rows/expert: 256-row tiles, exact multiples
+    (1100, 8, 2, 200, 264),      # 275 rows/expert: ragged row tails, K % 64 != 0, N % 256 != 0
+    (520, 8, 2, 320, 1000),      # 130 rows/expert: 128-row tiles
+    (130, 8, 3, 448, 72),        # ~49 rows/expert: 64-row tiles, N < one tile
+    (3, 8, 2, 64, 256),          # decode-like: a handful of rows
+    (2048, 32, 4, 192, 328),     # E = 32 with skew: tiny and empty experts
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("w_layout", ["k_contig", "n_contig"])
+@pytest.mark.parametrize("T,E,k,K,N", SHAPES)
+def test_s2s_gather_to_grouped(T, E, k, K, N, w_layout, dtype):
+    experts, (eid, idx, off) = _routing(T, E, k, seed=K + N, skew=2.0 if E == 32 else 0.0,
+                                        empty=(3,) if E == 32 else ())
+    g = torch.Generator().manual_seed(T)
+    X = torch.randn(T, K, generator=g).to(dtype)
+    Wp = (torch.randn(E, N, K, generator=g) * 0.1).to(dtype)          # parameter layout (E, out, in)
+    b = (torch.randn(E, N, generator=g)).to(dtype)
+    Wd = Wp.to(DEV).permute(0, 2, 1)
+    if w_layout == "n_contig":
+        Wd = Wd.contiguous()
+    want = oracle.scatter2scatter_ref(X.float(), Wp.permute(0, 2, 1).float(), eid, idx, k, b.float(), False, True)
+    got = ops.scatter2scatter(X.to(DEV), Wd, eid.to(DEV), idx.to(DEV), k, b=b.to(DEV), y_grouped=True,
+                              expert_offsets=off.to(DEV))
+    _close(got, want, scale=0.1 * K ** 0.5)
+
+
+@pytest.mark.parametrize("w_layout", ["k_contig", "n_contig"])
+@pytest.mark.parametrize("x_grouped,y_grouped", list(itertools.product([False, True], repeat=2)))
+def test_s2s_modes(x_grouped, y_grouped, w_layout):
+    T, E, k, K, N = 900, 8, 2, 256, 512
+    experts, (eid, idx, off) = _routing(T, E, k, seed=5, skew=1.0, empty=(6,))
+    g = torch.Generator().manual_seed(9)
+    fan = 1 if x_grouped else k
+    X = torch.randn(T * k // fan, K, generator=g).bfloat16()
+    Wp = (torch.randn(E, N, K, generator=g) * 0.1).bfloat16()
+    Wd = Wp.to(DEV).permute(0, 2, 1)
+    if w_layout == "n_contig":
+        Wd = Wd.contiguous()
+    want = oracle.scatter2scatter_ref(X.float(), Wp.permute(0, 2, 1).float(), eid, idx, fan, None, x_grouped, y_grouped)
+    out = torch.full((T * k, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    got = ops.scatter2scatter(X.to(DEV), Wd, eid.to(DEV), idx.to(DEV), fan, x_grouped=x_grouped,
+                              y_grouped=y_grouped, out=out, expert_offsets=off.to(DEV))
+    _close(got, want, scale=0.1 * K ** 0.5)
+    again = ops.scatter2scatter(X.to(DEV), Wd, eid.to(DEV), idx.to(DEV), fan, x_grouped=x_grouped,
+                                y_grouped=y_grouped, expert_offsets=off.to(DEV))
+    assert torch.equal(got, again)
+
+
+def test_s2s_strided_rows():
+    """X and Y that are column slices of wider buffers (row stride != width)."""
+    T, E, k, K, N = 600, 8, 2, 128, 256
+    experts, (eid, idx, off) = _routing(T, E, k, seed=1)
+    g = torch.Generator().manual_seed(2)
+    Xw = torch.randn(T, K + 64, generator=g).bfloat16()
+    W = (torch.randn(E, K, N, generator=g) * 0.1).bfloat16()
+    want = oracle.scatter2scatter_ref(Xw[:, 32:32 + K].float(), W.float(), eid, idx, k)
+    Yw = torch.zeros(T * k, N + 16, dtype=torch.bfloat16, device=DEV)
+    ops.scatter2scatter(Xw.to(DEV)[:, 32:32 + K], W.to(DEV), eid.to(DEV), idx.to(DEV), k, out=Yw[:, 8:8 + N])
+    _close(Yw[:, 8:8 + N], want, scale=0.1 * K ** 0.5)
+    assert not Yw[:, :8].any() and not Yw[:, 8 + N:].any()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("out_layout", ["param", "plain"])
+@pytest.mark.parametrize("T,E,k,K,N", [(4096, 8, 2, 512, 256), (1100, 8, 2, 200, 264), (130, 8, 3, 448, 72),
+                                       (2048, 32, 4, 192, 328), (700, 4, 1, 1024, 520)])
+def test_xty(T, E, k, K, N, out_layout, dtype):
+    experts, (eid, idx, off) = _routing(T, E, k, seed=N, skew=2.0 if E == 32 else 0.0, empty=(1,) if E == 32 else ())
+    g = torch.Generator().manual_seed(K)
+    L = T * k
+    X = torch.randn(L, K, generator=g).to(dtype)
+    DY = (torch.randn(L, N, generator=g) * 0.1).to(dtype)
+    DW_ref, Db_ref = oracle.group_bwd_W_ref(DY.float(), X.float(), off, E, has_bias=True)
+    rows = torch.diff(off, prepend=torch.zeros(1, dtype=torch.long)).max().item()
+    if out_layout == "param":
+        DW, Db = ops.group_bwd_W(DY.to(DEV), X.to(DEV), off.to(DEV), E, has_bias=True)
+        assert DW.permute(0, 2, 1).is_contiguous()
+    else:                                         # (E, K, N)-contiguous output through the raw op
+        DW = torch.full((E, K, N), float("nan"), dtype=dtype, device=DEV)
+        Db = torch.full((E, N), float("nan"), dtype=dtype, device=DEV)
+        ops._xty_launch(E, DW, Db, DY.to(DEV), X.to(DEV), off.to(DEV))
+    _close(DW, DW_ref, scale=0.1 * rows ** 0.5)
+    _close(Db, Db_ref, scale=0.1 * rows ** 0.5)
+    for e in (torch.diff(off, prepend=torch.zeros(1, dtype=torch.long)) == 0).nonzero().flatten().tolist():
+        assert not DW[e].any() and not Db[e].any()
