@@ -1,0 +1,181 @@
+"""Headline benchmark: Mixtral-shape bf16 MoE MLP forward+backward on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c1] [--no-cpu]
+
+One step = routing prep + GLUMLP forward + backward (dX, d gates, dW1, dW2) on synthetic inputs that
+are resident in HBM before the timed region.  Prints ONE JSON line.  The CPU figure next to it is the
+naive per-expert PyTorch path (the oracle) timed on the host cores on a reduced token count.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+os.environ.setdefault("SCATTERMOE_NO_HF_PATCH", "1")
+
+PEAK_BF16_TFLOPS = 2500.0        # MI355X dense bf16 MFMA peak
+PEAK_HBM_GBS = 8000.0
+
+# HBM bytes moved per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (KiB per dispatch, scaled by a copy kernel of known size); None until measured for a workload.
+MEASURED_TRAFFIC = {}
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c2")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-tokens", type=int, default=0, help="token count of the CPU sample (default T/16)")
+    return ap.parse_args()
+
+
+class TimedBackend:
+    """Wraps the launch layer and brackets every scatter2scatter launch with events on the launch stream."""
+
+    def __init__(self, inner, torch):
+        self.inner, self.torch, self.records, self.on = inner, torch, [], False
+
+    def __getattr__(self, name):
+        return getattr(self.inner, name)
+
+    def s2s(self, X, W, b, Y, eid, idx, off, k, x_grouped, y_grouped):
+        if not self.on:
+            return self.inner.s2s(X, W, b, Y, eid, idx, off, k, x_grouped, y_grouped)
+        a, c = self.torch.cuda.Event(enable_timing=True), self.torch.cuda.Event(enable_timing=True)
+        a.record()
+        self.inner.s2s(X, W, b, Y, eid, idx, off, k, x_grouped, y_grouped)
+        c.record()
+        self.records.append((a, c, 2.0 * eid.numel() * X.size(1) * Y.size(1), W.stride(1) == 1))
+
+
+def cpu_baseline(cfg, tokens, torch):
+    """Naive per-expert PyTorch path (oracle), fp32, forward + autograd backward, on `tokens` tokens."""
+    import oracle
+    from _inputs import make_inputs, scaled
+    small = scaled(cfg, T=tokens)
+    n1 = (2 if cfg.glu else 1) * cfg.f
+    t = make_inputs(small, weights=False)
+    g = torch.Generator().manual_seed(1)
+    W1 = torch.empty(cfg.E, n1, cfg.d).normal_(0, 0.02, generator=g).requires_grad_()
+    W2 = torch.empty(cfg.E, cfg.d, cfg.f).normal_(0, 0.02, generator=g).requires_grad_()
+    b1 = b2 = None
+    if cfg.bias:
+        b1 = torch.zeros(cfg.E, n1).requires_grad_()
+        b2 = torch.zeros(cfg.E, cfg.d).requires_grad_()
+    act = torch.nn.SiLU() if cfg.glu else torch.nn.GELU()
+    hidden = oracle.glu(act) if cfg.glu else act
+    x = t["x"].requires_grad_()
+    p = t["p"].requires_grad_()
+    t0 = time.perf_counter()
+    y = oracle.naive_expert_forward(x, p, t["experts"], W1, W2, hidden, b1, b2)
+    y.backward(t["dy"])
+    dt = time.perf_counter() - t0
+    return {"value": tokens / dt, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": "%s at T=%d of %d tokens (same d, f, E, k), fp32, 1 forward+backward, %.1f s; host has %d cpus"
+                      % (cfg.name, tokens, cfg.T, dt, os.cpu_count())}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build measures ONE GPU; --gpus %d is not supported "
+              "(no collective or multi-GPU code exists in this path)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from torch import nn
+    from _inputs import CONFIGS
+    from scattermoe_amd import _C
+    from scattermoe_amd.kernels import ops
+    from scattermoe_amd.mlp import GLUMLP, MLP
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    assert os.path.exists(_C.lib_path()), "libscattermoe_amd.so missing: run __graft_entry__.build()"
+    _C.load()
+    cfg = CONFIGS[args.workload]
+    dev = torch.device("cuda:0")
+    dtype = cfg.dtype
+
+    # synthetic inputs, generated on the device with a fixed seed; resident before timing starts
+    g = torch.Generator(device=dev).manual_seed(0)
+    logits = torch.randn(cfg.T, cfg.E, generator=g, device=dev)
+    if cfg.zipf_beta:
+        logits = logits - cfg.zipf_beta * 1.2 * torch.log(torch.arange(1, cfg.E + 1, device=dev).float())
+    p, experts = torch.topk(torch.softmax(logits, -1), cfg.k)
+    p = (p / p.sum(-1, keepdim=True)).to(dtype).requires_grad_()
+    x = torch.randn(cfg.T, cfg.d, generator=g, device=dev).to(dtype).requires_grad_()
+    dy = torch.randn(cfg.T, cfg.d, generator=g, device=dev).to(dtype)
+    cls = GLUMLP if cfg.glu else MLP
+    with torch.device(dev):
+        m = cls(cfg.d, cfg.f, cfg.E, cfg.k, bias=cfg.bias, activation=nn.SiLU() if cfg.glu else nn.GELU()).to(dtype)
+    if cfg.bias:
+        nn.init.normal_(m.experts.bias, std=0.02)
+        nn.init.normal_(m.output_experts.bias, std=0.02)
+    leaves = [x, p] + list(m.parameters())
+
+    timed = TimedBackend(ops._backend, torch)
+    ops._backend = timed
+
+    def step():
+        for t in leaves:
+            t.grad = None
+        y = m(x, p, experts)
+        y.backward(dy)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    timed.on = True
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    timed.on = False
+
+    L = cfg.T * cfg.k
+    flops_step = (18.0 if cfg.glu else 12.0) * L * cfg.d * cfg.f
+    ms = dt / args.steps * 1e3
+    tflops = flops_step / (ms * 1e-3) / 1e12
+
+    # dominant kernel: the MFMA scatter2scatter (forward flavour: weights with contiguous contraction axis)
+    fwd = [(a.elapsed_time(c), fl) for a, c, fl, kc in timed.records if kc]
+    allk = [(a.elapsed_time(c), fl) for a, c, fl, kc in timed.records]
+    sel = fwd if fwd else allk
+    k_ms = sum(t for t, _ in sel) / len(sel)
+    k_fl = sum(fl for _, fl in sel) / len(sel)
+    achieved = k_fl / (k_ms * 1e-3) / 1e12
+    roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": MEASURED_TRAFFIC.get(cfg.name),
+                "kernel": "s2s_mfma_kernel (scatter2scatter, K-contiguous weights)",
+                "launches_per_step": len(sel) // args.steps, "avg_launch_ms": round(k_ms, 4),
+                "avg_flop_per_launch": k_fl,
+                "all_s2s_launches_avg_tflops": round(sum(fl for _, fl in allk) / sum(t for t, _ in allk) / 1e9, 1)}
+
+    out = {
+        "metric": "moe_mlp_fwd_bwd_tokens_per_s", "value": round(cfg.T * args.steps / dt, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": {torch.bfloat16: "bf16", torch.float32: "f32", torch.float16: "f16"}[dtype], "data": "synthetic",
+        "config": {"workload": "%s: MoE MLP fwd+bwd T=%d d_model=%d d_ff=%d E=%d top_k=%d %s%s" % (
+            cfg.name, cfg.T, cfg.d, cfg.f, cfg.E, cfg.k, "SwiGLU" if cfg.glu else "GELU", " +bias" if cfg.bias else ""),
+            "tokens": cfg.T, "rows": L},
+        "tflops": round(tflops, 1), "frac_of_bf16_mfma_peak": round(tflops / PEAK_BF16_TFLOPS, 4),
+        "roofline": roofline,
+    }
+    if not args.no_cpu:
+        tokens = args.cpu_tokens or max(64, cfg.T // 16)
+        out["cpu_baseline"] = cpu_baseline(cfg, tokens, torch)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -22,16 +22,16 @@ def _run_pair(m_cpu, x, p, experts, dy, dtype, per_token=False):
     with torch.no_grad():                                    # oracle computes in fp32 on the rounded values
         for q, v in zip(m_cpu.parameters(), m_gpu.parameters()):
             q.copy_(v.float().cpu())
-    xg = x.to(dtype).to(DEV).requires_grad_()
-    pg = p.to(dtype).to(DEV).requires_grad_()
+    xg = x.to(dtype).to(DEV).detach().clone().requires_grad_()
+    pg = p.to(dtype).to(DEV).detach().clone().requires_grad_()
     params_g = [xg, pg, m_gpu.experts.weight, m_gpu.output_experts.weight]
     if m_gpu.experts.bias is not None:
         params_g += [m_gpu.experts.bias, m_gpu.output_experts.bias]
     y = m_gpu(xg, pg, experts.to(DEV))
     got = torch.autograd.grad(y, params_g, dy.to(dtype).to(DEV))
 
-    xc = x.to(dtype).float().requires_grad_()
-    pc = p.to(dtype).float().requires_grad_()
+    xc = x.to(dtype).float().detach().clone().requires_grad_()
+    pc = p.to(dtype).float().detach().clone().requires_grad_()
     params_c = [xc, pc, m_cpu.experts.weight, m_cpu.output_experts.weight]
     if m_cpu.experts.bias is not None:
         params_c += [m_cpu.experts.bias, m_cpu.output_experts.bias]
