@@ -32,6 +32,9 @@ enum { SMOE_F32 = 0, SMOE_BF16 = 1, SMOE_F16 = 2 };
 /* element types of the unsorted expert-index tensor handed to smoe_route */
 enum { SMOE_I64 = 0, SMOE_I32 = 1, SMOE_I16 = 2, SMOE_U8 = 3 };
 
+/* activations of the gated linear unit kernels */
+enum { SMOE_ACT_SILU = 0 };
+
 /* argument errors */
 enum {
   SMOE_ERR_NULL = -1,      /* a required pointer is NULL */
@@ -117,6 +120,35 @@ int smoe_groupXtY(const void* DY, int64_t sdym, int64_t sdyn,
                   void* Db, int64_t sdbe, int64_t sdbn,
                   const int64_t* off, int64_t L, int64_t K, int64_t N, int E,
                   int dtype, void* stream);
+
+/*
+ * Gate-weighted sum of the k expert outputs of each token:  out[t,:] = sum_j gates[t,j] * Y[t*k+j,:].
+ * Replaces the batched matmul `gates.unsqueeze(1) @ output_expanded` of ParallelLinear.forward
+ * (scattermoe/parallel_experts.py:44-46).  Y (T*k, N) row stride sym (columns contiguous), gates (T,k)
+ * strides sgt,sgk, out (T,N) row stride som.  fp32 accumulation in slot order, one rounding.
+ */
+int smoe_combine(const void* Y, int64_t sym, const void* gates, int64_t sgt, int64_t sgk, void* out, int64_t som,
+                 int64_t T, int k, int64_t N, int dtype, void* stream);
+
+/*
+ * Gradient of the gates:  dgates[t,j] = < Y[t*k+j,:], dOut[t,:] >.
+ * Replaces `output_expanded @ grad_out.unsqueeze(-1)` of ParallelLinear.backward
+ * (scattermoe/parallel_experts.py:76-82).  Y (T*k, N) row stride sym, dOut (T,N) row stride sdm,
+ * dgates (T,k) strides sgt,sgk.
+ */
+int smoe_gate_grad(const void* Y, int64_t sym, const void* dOut, int64_t sdm, void* dgates, int64_t sgt, int64_t sgk,
+                   int64_t T, int k, int64_t N, int dtype, void* stream);
+
+/*
+ * Gated linear unit of GLUMLP in one pass:  h = act(pre[:, f:2f]) * pre[:, 0:f]   (first half linear,
+ * second half activated), replacing chunk + activation + multiply of scattermoe/mlp.py:81-87, and its
+ * gradient  dpre[:, 0:f] = dh * act(g),  dpre[:, f:2f] = dh * lin * act'(g)  that autograd derives from it.
+ * pre / dpre (rows, 2f) row strides spm / sdpm, h / dh (rows, f) row strides shm / sdhm; `act` = SMOE_ACT_*.
+ */
+int smoe_glu_fwd(const void* pre, int64_t spm, void* h, int64_t shm, int64_t rows, int64_t f, int act, int dtype,
+                 void* stream);
+int smoe_glu_bwd(const void* pre, int64_t spm, const void* dh, int64_t sdhm, void* dpre, int64_t sdpm, int64_t rows,
+                 int64_t f, int act, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

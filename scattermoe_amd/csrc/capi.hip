@@ -106,4 +106,50 @@ int smoe_groupXtY(const void* DY, int64_t sdym, int64_t sdyn, const void* X, int
   return launch_xty_generic(a, dtype, (hipStream_t)stream);
 }
 
+int smoe_combine(const void* Y, int64_t sym, const void* gates, int64_t sgt, int64_t sgk, void* out, int64_t som,
+                 int64_t T, int k, int64_t N, int dtype, void* stream) {
+  g_err[0] = 0;
+  if (!dtype_ok(dtype)) { set_error("smoe_combine: unknown dtype %d", dtype); return SMOE_ERR_DTYPE; }
+  if (T < 0 || k <= 0 || N < 0) { set_error("smoe_combine: bad sizes"); return SMOE_ERR_SHAPE; }
+  if (T > 0x7fffffffLL || N > 0x7fffffffLL) { set_error("smoe_combine: size beyond int32"); return SMOE_ERR_RANGE; }
+  if (T == 0 || N == 0) return 0;
+  if (!Y || !gates || !out) { set_error("smoe_combine: NULL pointer"); return SMOE_ERR_NULL; }
+  return launch_combine(Y, sym, gates, sgt, sgk, out, som, T, k, (int)N, dtype, (hipStream_t)stream);
+}
+
+int smoe_gate_grad(const void* Y, int64_t sym, const void* dOut, int64_t sdm, void* dgates, int64_t sgt, int64_t sgk,
+                   int64_t T, int k, int64_t N, int dtype, void* stream) {
+  g_err[0] = 0;
+  if (!dtype_ok(dtype)) { set_error("smoe_gate_grad: unknown dtype %d", dtype); return SMOE_ERR_DTYPE; }
+  if (T < 0 || k <= 0 || N < 0) { set_error("smoe_gate_grad: bad sizes"); return SMOE_ERR_SHAPE; }
+  if (T > 0x7fffffffLL || N > 0x7fffffffLL) { set_error("smoe_gate_grad: size beyond int32"); return SMOE_ERR_RANGE; }
+  if (T == 0) return 0;
+  if (!dgates || (N > 0 && (!Y || !dOut))) { set_error("smoe_gate_grad: NULL pointer"); return SMOE_ERR_NULL; }
+  return launch_gate_grad(Y, sym, dOut, sdm, dgates, sgt, sgk, T, k, (int)N, dtype, (hipStream_t)stream);
+}
+
+int smoe_glu_fwd(const void* pre, int64_t spm, void* h, int64_t shm, int64_t rows, int64_t f, int act, int dtype,
+                 void* stream) {
+  g_err[0] = 0;
+  if (!dtype_ok(dtype)) { set_error("smoe_glu_fwd: unknown dtype %d", dtype); return SMOE_ERR_DTYPE; }
+  if (rows < 0 || f < 0) { set_error("smoe_glu_fwd: bad sizes"); return SMOE_ERR_SHAPE; }
+  if (act != SMOE_ACT_SILU) { set_error("smoe_glu_fwd: unknown activation %d", act); return SMOE_ERR_SHAPE; }
+  if (f > 0x3fffffffLL) { set_error("smoe_glu_fwd: size beyond int32"); return SMOE_ERR_RANGE; }
+  if (rows == 0 || f == 0) return 0;
+  if (!pre || !h) { set_error("smoe_glu_fwd: NULL pointer"); return SMOE_ERR_NULL; }
+  return launch_glu_fwd(pre, spm, h, shm, rows, (int)f, act, dtype, (hipStream_t)stream);
+}
+
+int smoe_glu_bwd(const void* pre, int64_t spm, const void* dh, int64_t sdhm, void* dpre, int64_t sdpm, int64_t rows,
+                 int64_t f, int act, int dtype, void* stream) {
+  g_err[0] = 0;
+  if (!dtype_ok(dtype)) { set_error("smoe_glu_bwd: unknown dtype %d", dtype); return SMOE_ERR_DTYPE; }
+  if (rows < 0 || f < 0) { set_error("smoe_glu_bwd: bad sizes"); return SMOE_ERR_SHAPE; }
+  if (act != SMOE_ACT_SILU) { set_error("smoe_glu_bwd: unknown activation %d", act); return SMOE_ERR_SHAPE; }
+  if (f > 0x3fffffffLL) { set_error("smoe_glu_bwd: size beyond int32"); return SMOE_ERR_RANGE; }
+  if (rows == 0 || f == 0) return 0;
+  if (!pre || !dh || !dpre) { set_error("smoe_glu_bwd: NULL pointer"); return SMOE_ERR_NULL; }
+  return launch_glu_bwd(pre, spm, dh, sdhm, dpre, sdpm, rows, (int)f, act, dtype, (hipStream_t)stream);
+}
+
 }  // extern "C"

@@ -106,6 +106,15 @@ int launch_group(const GroupArgs& a, int dtype, hipStream_t st);
 bool try_s2s_mfma(const S2SArgs& a, int dtype, hipStream_t st, int& rc);
 bool try_xty_mfma(const XtYArgs& a, int dtype, hipStream_t st, int& rc);
 
+int launch_combine(const void* Y, int64_t sy, const void* G, int64_t sgt, int64_t sgk, void* O, int64_t so,
+                   int64_t Tn, int k, int N, int dtype, hipStream_t st);
+int launch_gate_grad(const void* Y, int64_t sy, const void* D, int64_t sd, void* DG, int64_t sgt, int64_t sgk,
+                     int64_t Tn, int k, int N, int dtype, hipStream_t st);
+int launch_glu_fwd(const void* pre, int64_t sp, void* h, int64_t sh, int64_t rows, int f, int act, int dtype,
+                   hipStream_t st);
+int launch_glu_bwd(const void* pre, int64_t sp, const void* dh, int64_t sdh, void* dpre, int64_t sdp, int64_t rows,
+                   int f, int act, int dtype, hipStream_t st);
+
 int launch_route(const void* expert_idxs, int idx_dtype, int64_t L, int E, int64_t* eid_out,
                  int64_t* idx_out, int64_t* off_out, void* ws, hipStream_t st);
 size_t route_workspace_bytes(int64_t L, int E);

@@ -1,0 +1,212 @@
+// HBM-bound passes around the expert GEMMs, each one read + one write instead of a library bmm or a
+// chain of elementwise launches:
+//   combine    out[t,:]  = sum_j gates[t,j] * Y[t*k+j,:]        (reference: parallel_experts.py:44-46, a bmm)
+//   gate_grad  dg[t,j]   = <Y[t*k+j,:], dOut[t,:]>              (reference: parallel_experts.py:79, a bmm)
+//   glu_fwd    h         = act(pre[:, f:]) * pre[:, :f]          (reference: mlp.py:81-87, chunk + act + mul)
+//   glu_bwd    dpre      = [dh * act(g), dh * lin * act'(g)]     (autograd of the same expression)
+// All arithmetic in fp32, one rounding to the tensor dtype on store.
+#include "common.hpp"
+
+namespace smoe {
+
+template <typename T> struct Pack { static constexpr int n = 16 / sizeof(T); T v[16 / sizeof(T)]; };
+
+// ---- combine -------------------------------------------------------------------------------------------
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void combine_kernel(const T* __restrict__ Y, int64_t sy, const T* __restrict__ G,
+                                                     int64_t sgt, int64_t sgk, T* __restrict__ O, int64_t so,
+                                                     int k, int N) {
+  const int64_t t = blockIdx.x;
+  const T* y0 = Y + t * k * sy;
+  if (VEC) {
+    typedef Pack<T> P;
+    for (int c = threadIdx.x; c < N / P::n; c += 256) {
+      float acc[P::n];
+#pragma unroll
+      for (int q = 0; q < P::n; ++q) acc[q] = 0.0f;
+      for (int j = 0; j < k; ++j) {
+        const float g = to_f32(G[t * sgt + j * sgk]);
+        const P x = *(const P*)(y0 + j * sy + (int64_t)c * P::n);
+#pragma unroll
+        for (int q = 0; q < P::n; ++q) acc[q] = fmaf(g, to_f32(x.v[q]), acc[q]);
+      }
+      P o;
+#pragma unroll
+      for (int q = 0; q < P::n; ++q) o.v[q] = from_f32<T>(acc[q]);
+      *(P*)(O + t * so + (int64_t)c * P::n) = o;
+    }
+  } else {
+    for (int n = threadIdx.x; n < N; n += 256) {
+      float acc = 0.0f;
+      for (int j = 0; j < k; ++j) acc = fmaf(to_f32(G[t * sgt + j * sgk]), to_f32(y0[j * sy + n]), acc);
+      O[t * so + n] = from_f32<T>(acc);
+    }
+  }
+}
+
+// ---- gate gradient --------------------------------------------------------------------------------------
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void gate_grad_kernel(const T* __restrict__ Y, int64_t sy, const T* __restrict__ D,
+                                                       int64_t sd, T* __restrict__ DG, int64_t sgt, int64_t sgk,
+                                                       int k, int N) {
+  __shared__ float part[4];
+  const int64_t t = blockIdx.x;
+  const int lane = lane_id(), wave = threadIdx.x >> 6;
+  for (int j = 0; j < k; ++j) {
+    const T* y = Y + (t * k + j) * sy;
+    const T* d = D + t * sd;
+    float acc = 0.0f;
+    if (VEC) {
+      typedef Pack<T> P;
+      for (int c = threadIdx.x; c < N / P::n; c += 256) {
+        const P a = *(const P*)(y + (int64_t)c * P::n);
+        const P b = *(const P*)(d + (int64_t)c * P::n);
+#pragma unroll
+        for (int q = 0; q < P::n; ++q) acc = fmaf(to_f32(a.v[q]), to_f32(b.v[q]), acc);
+      }
+    } else {
+      for (int n = threadIdx.x; n < N; n += 256) acc = fmaf(to_f32(y[n]), to_f32(d[n]), acc);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+    if (lane == 0) part[wave] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) DG[t * sgt + j * sgk] = from_f32<T>((part[0] + part[1]) + (part[2] + part[3]));
+    __syncthreads();
+  }
+}
+
+// ---- gated linear unit -----------------------------------------------------------------------------------
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + __expf(-x)); }
+__device__ __forceinline__ float act_f(int act, float g) { (void)act; return g * sigmoidf_(g); }
+__device__ __forceinline__ float act_df(int act, float g) {
+  (void)act;
+  const float s = sigmoidf_(g);
+  return s * (1.0f + g * (1.0f - s));
+}
+
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void glu_fwd_kernel(const T* __restrict__ pre, int64_t sp, T* __restrict__ h,
+                                                     int64_t sh, int64_t rows, int f, int act) {
+  constexpr int W = VEC ? Pack<T>::n : 1;
+  const int64_t per_row = f / W;
+  const int64_t total = rows * per_row;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / per_row, c = (i % per_row) * W;
+    if (VEC) {
+      typedef Pack<T> P;
+      const P lin = *(const P*)(pre + r * sp + c);
+      const P gat = *(const P*)(pre + r * sp + f + c);
+      P o;
+#pragma unroll
+      for (int q = 0; q < P::n; ++q) o.v[q] = from_f32<T>(act_f(act, to_f32(gat.v[q])) * to_f32(lin.v[q]));
+      *(P*)(h + r * sh + c) = o;
+    } else {
+      h[r * sh + c] = from_f32<T>(act_f(act, to_f32(pre[r * sp + f + c])) * to_f32(pre[r * sp + c]));
+    }
+  }
+}
+
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void glu_bwd_kernel(const T* __restrict__ pre, int64_t sp, const T* __restrict__ dh,
+                                                     int64_t sdh, T* __restrict__ dpre, int64_t sdp, int64_t rows,
+                                                     int f, int act) {
+  constexpr int W = VEC ? Pack<T>::n : 1;
+  const int64_t per_row = f / W;
+  const int64_t total = rows * per_row;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / per_row, c = (i % per_row) * W;
+    if (VEC) {
+      typedef Pack<T> P;
+      const P lin = *(const P*)(pre + r * sp + c);
+      const P gat = *(const P*)(pre + r * sp + f + c);
+      const P d = *(const P*)(dh + r * sdh + c);
+      P ol, og;
+#pragma unroll
+      for (int q = 0; q < P::n; ++q) {
+        const float g = to_f32(gat.v[q]), dv = to_f32(d.v[q]);
+        ol.v[q] = from_f32<T>(dv * act_f(act, g));
+        og.v[q] = from_f32<T>(dv * to_f32(lin.v[q]) * act_df(act, g));
+      }
+      *(P*)(dpre + r * sdp + c) = ol;
+      *(P*)(dpre + r * sdp + f + c) = og;
+    } else {
+      const float g = to_f32(pre[r * sp + f + c]), dv = to_f32(dh[r * sdh + c]);
+      dpre[r * sdp + c] = from_f32<T>(dv * act_f(act, g));
+      dpre[r * sdp + f + c] = from_f32<T>(dv * to_f32(pre[r * sp + c]) * act_df(act, g));
+    }
+  }
+}
+
+static bool al16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+static unsigned ew_grid(int64_t total) {
+  int64_t b = cdiv64(total, 256);
+  return (unsigned)(b > 256 * 32 ? 256 * 32 : (b < 1 ? 1 : b));
+}
+
+template <typename T>
+static int combine_t(const void* Y, int64_t sy, const void* G, int64_t sgt, int64_t sgk, void* O, int64_t so,
+                     int64_t Tn, int k, int N, hipStream_t st) {
+  constexpr int vn = 16 / sizeof(T);
+  const bool vec = N % vn == 0 && sy % vn == 0 && so % vn == 0 && al16(Y) && al16(O);
+  if (vec) hipLaunchKernelGGL((combine_kernel<T, true>), dim3((unsigned)Tn), dim3(256), 0, st, (const T*)Y, sy, (const T*)G, sgt, sgk, (T*)O, so, k, N);
+  else hipLaunchKernelGGL((combine_kernel<T, false>), dim3((unsigned)Tn), dim3(256), 0, st, (const T*)Y, sy, (const T*)G, sgt, sgk, (T*)O, so, k, N);
+  return launch_status("combine_kernel");
+}
+
+template <typename T>
+static int gate_grad_t(const void* Y, int64_t sy, const void* D, int64_t sd, void* DG, int64_t sgt, int64_t sgk,
+                       int64_t Tn, int k, int N, hipStream_t st) {
+  constexpr int vn = 16 / sizeof(T);
+  const bool vec = N % vn == 0 && sy % vn == 0 && sd % vn == 0 && al16(Y) && al16(D);
+  if (vec) hipLaunchKernelGGL((gate_grad_kernel<T, true>), dim3((unsigned)Tn), dim3(256), 0, st, (const T*)Y, sy, (const T*)D, sd, (T*)DG, sgt, sgk, k, N);
+  else hipLaunchKernelGGL((gate_grad_kernel<T, false>), dim3((unsigned)Tn), dim3(256), 0, st, (const T*)Y, sy, (const T*)D, sd, (T*)DG, sgt, sgk, k, N);
+  return launch_status("gate_grad_kernel");
+}
+
+template <typename T>
+static int glu_fwd_t(const void* pre, int64_t sp, void* h, int64_t sh, int64_t rows, int f, int act, hipStream_t st) {
+  constexpr int vn = 16 / sizeof(T);
+  const bool vec = f % vn == 0 && sp % vn == 0 && sh % vn == 0 && al16(pre) && al16(h);
+  const int64_t total = rows * (f / (vec ? vn : 1));
+  if (vec) hipLaunchKernelGGL((glu_fwd_kernel<T, true>), dim3(ew_grid(total)), dim3(256), 0, st, (const T*)pre, sp, (T*)h, sh, rows, f, act);
+  else hipLaunchKernelGGL((glu_fwd_kernel<T, false>), dim3(ew_grid(total)), dim3(256), 0, st, (const T*)pre, sp, (T*)h, sh, rows, f, act);
+  return launch_status("glu_fwd_kernel");
+}
+
+template <typename T>
+static int glu_bwd_t(const void* pre, int64_t sp, const void* dh, int64_t sdh, void* dpre, int64_t sdp, int64_t rows,
+                     int f, int act, hipStream_t st) {
+  constexpr int vn = 16 / sizeof(T);
+  const bool vec = f % vn == 0 && sp % vn == 0 && sdh % vn == 0 && sdp % vn == 0 && al16(pre) && al16(dh) && al16(dpre);
+  const int64_t total = rows * (f / (vec ? vn : 1));
+  if (vec) hipLaunchKernelGGL((glu_bwd_kernel<T, true>), dim3(ew_grid(total)), dim3(256), 0, st, (const T*)pre, sp, (const T*)dh, sdh, (T*)dpre, sdp, rows, f, act);
+  else hipLaunchKernelGGL((glu_bwd_kernel<T, false>), dim3(ew_grid(total)), dim3(256), 0, st, (const T*)pre, sp, (const T*)dh, sdh, (T*)dpre, sdp, rows, f, act);
+  return launch_status("glu_bwd_kernel");
+}
+
+#define SMOE_DISPATCH(dtype, CALL)                                              \
+  switch (dtype) {                                                              \
+    case SMOE_F32: { typedef float T; return CALL; }                            \
+    case SMOE_BF16: { typedef bf16_t T; return CALL; }                          \
+    case SMOE_F16: { typedef f16_t T; return CALL; }                            \
+    default: set_error("unknown dtype %d", dtype); return SMOE_ERR_DTYPE;       \
+  }
+
+int launch_combine(const void* Y, int64_t sy, const void* G, int64_t sgt, int64_t sgk, void* O, int64_t so,
+                   int64_t Tn, int k, int N, int dtype, hipStream_t st) {
+  SMOE_DISPATCH(dtype, combine_t<T>(Y, sy, G, sgt, sgk, O, so, Tn, k, N, st));
+}
+int launch_gate_grad(const void* Y, int64_t sy, const void* D, int64_t sd, void* DG, int64_t sgt, int64_t sgk,
+                     int64_t Tn, int k, int N, int dtype, hipStream_t st) {
+  SMOE_DISPATCH(dtype, gate_grad_t<T>(Y, sy, D, sd, DG, sgt, sgk, Tn, k, N, st));
+}
+int launch_glu_fwd(const void* pre, int64_t sp, void* h, int64_t sh, int64_t rows, int f, int act, int dtype, hipStream_t st) {
+  SMOE_DISPATCH(dtype, glu_fwd_t<T>(pre, sp, h, sh, rows, f, act, st));
+}
+int launch_glu_bwd(const void* pre, int64_t sp, const void* dh, int64_t sdh, void* dpre, int64_t sdp, int64_t rows,
+                   int f, int act, int dtype, hipStream_t st) {
+  SMOE_DISPATCH(dtype, glu_bwd_t<T>(pre, sp, dh, sdh, dpre, sdp, rows, f, act, st));
+}
+
+}  // namespace smoe

@@ -90,6 +90,47 @@ class HipBackend:
         _C.check(rc, "smoe_groupXtY")
 
 
+    @staticmethod
+    def combine(Y, gates, out, k):
+        _C.require_gpu(Y, "combine")
+        lib = _C.load()
+        with torch.cuda.device(Y.device):
+            rc = lib.smoe_combine(_C.ptr(Y), Y.stride(0), _C.ptr(gates), gates.stride(0), gates.stride(1),
+                                  _C.ptr(out), out.stride(0), out.size(0), k, Y.size(1),
+                                  _C.float_code(Y.dtype), _C.stream_ptr(Y.device))
+        _C.check(rc, "smoe_combine")
+
+    @staticmethod
+    def gate_grad(Y, d_out, d_gates, k):
+        _C.require_gpu(Y, "gate_grad")
+        lib = _C.load()
+        with torch.cuda.device(Y.device):
+            rc = lib.smoe_gate_grad(_C.ptr(Y), Y.stride(0), _C.ptr(d_out), d_out.stride(0),
+                                    _C.ptr(d_gates), d_gates.stride(0), d_gates.stride(1),
+                                    d_out.size(0), k, Y.size(1), _C.float_code(Y.dtype),
+                                    _C.stream_ptr(Y.device))
+        _C.check(rc, "smoe_gate_grad")
+
+    @staticmethod
+    def glu_fwd(pre, h, act):
+        _C.require_gpu(pre, "glu_fwd")
+        lib = _C.load()
+        with torch.cuda.device(pre.device):
+            rc = lib.smoe_glu_fwd(_C.ptr(pre), pre.stride(0), _C.ptr(h), h.stride(0), pre.size(0), h.size(1),
+                                  act, _C.float_code(pre.dtype), _C.stream_ptr(pre.device))
+        _C.check(rc, "smoe_glu_fwd")
+
+    @staticmethod
+    def glu_bwd(pre, dh, dpre, act):
+        _C.require_gpu(pre, "glu_bwd")
+        lib = _C.load()
+        with torch.cuda.device(pre.device):
+            rc = lib.smoe_glu_bwd(_C.ptr(pre), pre.stride(0), _C.ptr(dh), dh.stride(0), _C.ptr(dpre),
+                                  dpre.stride(0), pre.size(0), dh.size(1), act, _C.float_code(pre.dtype),
+                                  _C.stream_ptr(pre.device))
+        _C.check(rc, "smoe_glu_bwd")
+
+
 _backend = HipBackend()
 
 
@@ -239,3 +280,51 @@ def _group_launch(A, Y, coeff, fan_out, idx):
 def group_compileable(A: torch.Tensor, K: int, N: int, Y: torch.Tensor, coeff: Optional[torch.Tensor],
                       has_coeff: bool, fan_out: int, sorted_expert_idxs: torch.Tensor) -> None:
     _group_launch(A, Y, coeff if has_coeff else None, fan_out, sorted_expert_idxs)
+
+
+# ------------------------------------------------------------------------------------------------
+# fused passes around the expert GEMMs
+# ------------------------------------------------------------------------------------------------
+ACT_SILU = 0
+
+
+def _rows_contiguous(t):
+    return t if t.stride(-1) == 1 else t.contiguous()
+
+
+def combine(expanded, gates):
+    """out[t] = sum_j gates[t, j] * expanded[t, j]  for expanded (T, k, N) -> (T, N)
+    (the bmm of reference parallel_experts.py:44-46 as one HBM pass)."""
+    T, k, N = expanded.shape
+    assert gates.shape == (T, k)
+    Y = _rows_contiguous(expanded.reshape(T * k, N))
+    out = torch.empty((T, N), dtype=expanded.dtype, device=expanded.device)
+    _backend.combine(Y, gates.to(expanded.dtype), out, k)
+    return out
+
+
+def gate_grad(expanded, grad_out):
+    """d_gates[t, j] = <expanded[t, j], grad_out[t]>  (the bmm of reference parallel_experts.py:79)."""
+    T, k, N = expanded.shape
+    assert grad_out.shape == (T, N)
+    Y = _rows_contiguous(expanded.reshape(T * k, N))
+    d_gates = torch.empty((T, k), dtype=expanded.dtype, device=expanded.device)
+    _backend.gate_grad(Y, _rows_contiguous(grad_out), d_gates, k)
+    return d_gates
+
+
+def glu_fwd(pre, act=ACT_SILU):
+    """h = act(pre[:, f:]) * pre[:, :f] for pre (rows, 2f)."""
+    assert pre.dim() == 2 and pre.size(1) % 2 == 0
+    pre = _rows_contiguous(pre)
+    h = torch.empty((pre.size(0), pre.size(1) // 2), dtype=pre.dtype, device=pre.device)
+    _backend.glu_fwd(pre, h, act)
+    return h
+
+
+def glu_bwd(pre, dh, act=ACT_SILU):
+    pre, dh = _rows_contiguous(pre), _rows_contiguous(dh)
+    assert dh.size(0) == pre.size(0) and 2 * dh.size(1) == pre.size(1)
+    dpre = torch.empty_like(pre)
+    _backend.glu_bwd(pre, dh, dpre, act)
+    return dpre

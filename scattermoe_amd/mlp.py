@@ -4,7 +4,23 @@
 import torch
 from torch import nn
 
+from .kernels import ops
 from .parallel_experts import ParallelExperts, flatten_sort_count
+
+
+class _FusedGLU(torch.autograd.Function):
+    """act(second half) * first half in one pass each way (saves the pre-activation, recomputes act)."""
+
+    @staticmethod
+    def forward(ctx, pre, act):
+        ctx.save_for_backward(pre)
+        ctx.act = act
+        return ops.glu_fwd(pre, act)
+
+    @staticmethod
+    def backward(ctx, dh):
+        (pre,) = ctx.saved_tensors
+        return ops.glu_bwd(pre, dh, ctx.act), None
 
 
 class _SparseMLP(nn.Module):
@@ -58,5 +74,7 @@ class GLUMLP(_SparseMLP):
         super().__init__(input_size, hidden_size, num_experts, top_k, bias, activation)
 
     def _hidden(self, pre):
+        if type(self.activation) is nn.SiLU and pre.dim() == 2:
+            return _FusedGLU.apply(pre, ops.ACT_SILU)
         lin, gate = pre.chunk(2, dim=-1)
         return self.activation(gate) * lin

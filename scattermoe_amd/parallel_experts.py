@@ -42,11 +42,6 @@ def flatten_sort_count(expert_idxs: torch.Tensor, num_experts: int):
 flatten_and_sort = flatten_sort_count
 
 
-def _combine(gates, expanded):
-    # (T, 1, k) @ (T, k, N) -> (T, N): gate-weighted sum over the k expert outputs of a token
-    return torch.bmm(gates.unsqueeze(1), expanded).squeeze(1)
-
-
 class ParallelLinear(torch.autograd.Function):
     """y = scatter2scatter(x, W[, b]) [combined with gates]; backward via group / groupXtY / scatter2scatter."""
 
@@ -66,7 +61,7 @@ class ParallelLinear(torch.autograd.Function):
                 result, kept = expanded, None
             else:
                 kept = expanded.view(gates.size(0), gates.size(1), expanded.size(-1))
-                result = _combine(gates, kept)
+                result = ops.combine(kept, gates)
         ctx.save_for_backward(x, expert_weights, expert_biases, sorted_expert_idxs,
                               sorted_scattered_idxs, expert_offsets, gates, kept)
         ctx.k, ctx.grouped_in, ctx.grouped_out = k, grouped_in, grouped_out
@@ -88,8 +83,8 @@ class ParallelLinear(torch.autograd.Function):
             coeff, coeff_fan, dy_buf = None, 1, None
             if gates is not None:
                 if need_g:
-                    # (T, k, N) @ (T, N, 1) -> (T, k): row dots of every expert output with dY
-                    d_gates = torch.bmm(kept, grad_out.unsqueeze(-1)).squeeze(-1)
+                    # (T, k): row dots of every expert output with dY
+                    d_gates = ops.gate_grad(kept, grad_out)
                 coeff, coeff_fan = gates.reshape(-1), gates.size(1)
                 dy_buf = kept.view(-1, kept.size(-1))   # its contents are dead once d_gates exists
 

@@ -30,3 +30,22 @@ class OracleBackend:
         DW.copy_(dw)
         if Db is not None:
             Db.copy_(db)
+
+    @staticmethod
+    def combine(Y, gates, out, k):
+        out.copy_((Y.view(out.size(0), k, -1).float() * gates.float().unsqueeze(-1)).sum(1))
+
+    @staticmethod
+    def gate_grad(Y, d_out, d_gates, k):
+        d_gates.copy_((Y.view(d_out.size(0), k, -1).float() * d_out.float().unsqueeze(1)).sum(-1))
+
+    @staticmethod
+    def glu_fwd(pre, h, act):
+        lin, gate = pre.float().chunk(2, dim=-1)
+        h.copy_(torch.nn.functional.silu(gate) * lin)
+
+    @staticmethod
+    def glu_bwd(pre, dh, dpre, act):
+        lin, gate = pre.float().chunk(2, dim=-1)
+        s = torch.sigmoid(gate)
+        dpre.copy_(torch.cat([dh.float() * gate * s, dh.float() * lin * s * (1 + gate * (1 - s))], dim=-1))

@@ -175,3 +175,37 @@ def test_group_bwd_W(T, E, k, K, N, dtype):
         assert not DW[e].any() and not Db[e].any()                        # written as exact zeros
     DW2, _ = ops.group_bwd_W(DY.to(DEV), X.to(DEV), off.to(DEV), E, has_bias=False)
     assert torch.equal(DW2, DW)                                           # fixed summation order
+
+
+# ---------------------------------------------------------------------------------------------------
+# fused passes: combine, gate gradient, gated linear unit
+# ---------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,k,N", [(1, 2, 128), (300, 3, 100), (1024, 2, 4096), (77, 8, 264), (50, 1, 64)])
+def test_combine_and_gate_grad(T, k, N, dtype):
+    g = torch.Generator().manual_seed(T + N)
+    Y = torch.randn(T, k, N, generator=g).to(dtype)
+    gates = torch.rand(T, k, generator=g).to(dtype)
+    dO = torch.randn(T, N, generator=g).to(dtype)
+    want = (Y.float() * gates.float().unsqueeze(-1)).sum(1)
+    got = ops.combine(Y.to(DEV), gates.to(DEV))
+    _close(got, want, dtype, scale=k ** 0.5)
+    want_g = (Y.float() * dO.float().unsqueeze(1)).sum(-1)
+    got_g = ops.gate_grad(Y.to(DEV), dO.to(DEV))
+    _close(got_g, want_g, dtype, scale=N ** 0.5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,f", [(1, 128), (333, 100), (4096, 768), (64, 2880)])
+def test_glu_fwd_bwd(rows, f, dtype):
+    g = torch.Generator().manual_seed(rows + f)
+    pre = torch.randn(rows, 2 * f, generator=g).to(dtype)
+    dh = torch.randn(rows, f, generator=g).to(dtype)
+    ref_in = pre.float().requires_grad_()
+    lin, gate = ref_in.chunk(2, dim=-1)
+    h_ref = torch.nn.functional.silu(gate) * lin
+    h_ref.backward(dh.float())
+    h = ops.glu_fwd(pre.to(DEV))
+    dpre = ops.glu_bwd(pre.to(DEV), dh.to(DEV))
+    _close(h, h_ref.detach(), dtype, scale=0.1)
+    _close(dpre, ref_in.grad, dtype, scale=0.1)
