@@ -23,7 +23,6 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
 static constexpr int BK = 64;               // contraction slice per stage
-static constexpr int kTrPad = 64;           // bytes of padding per row of a transposed LDS tile
 
 template <typename T> struct Mfma;
 template <> struct Mfma<bf16_t> {
@@ -49,90 +48,148 @@ template <> struct Mfma<f16_t> {
 
 typedef __attribute__((address_space(3))) char lds_char;
 
+__device__ __forceinline__ unsigned lds_address(const char* p) {
+  return (unsigned)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
+}
+__device__ __forceinline__ unsigned wave_uniform_id() {
+  return __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+}
 __device__ __forceinline__ i32x4 lds_read16(const char* p) { return *(const i32x4*)p; }
 __device__ __forceinline__ void lds_write16(char* p, i32x4 v) { *(i32x4*)p = v; }
 __device__ __forceinline__ s16x4 lds_read_tr(const char* p) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p);
 }
 
-// ---- operand with contiguous contraction axis: LDS tile [EXT][64], 128 B per row, swizzled ----------
-__device__ __forceinline__ int direct_off(int row, int chunk) {
-  const int s = (row & 7) ^ ((row >> 3) & 1);
-  return row * 128 + ((chunk ^ s) << 4);
+typedef __attribute__((address_space(3))) void lds_void_t;
+typedef __attribute__((address_space(1))) const void glb_void_t;
+
+// 16 bytes per lane straight from global memory into LDS: lane i of the wave lands at dst + 16*i.
+// Issued as inline assembly on purpose: for the builtin the compiler assumes that every later LDS read
+// may alias the in-flight transfer and waits for it (vmcnt(0)) before the first ds_read, which would
+// serialise the prefetch of slice k+1 with the MFMAs of slice k.  The main loop waits explicitly instead.
+// `lds_addr` is the wave-uniform byte address inside the workgroup's LDS allocation.
+__device__ __forceinline__ void load_to_lds16(const char* src, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+               :
+               : "s"(lds_addr), "v"(src)
+               : "memory", "m0");
 }
+
+// Both operand kinds fill a 64-deep LDS tile of EXT*128 bytes in LINEAR order of 16-byte pieces: piece
+// p = j*NT + t is copied by thread t in round j (a wave's 64 pieces are contiguous, which is what the
+// direct-to-LDS load needs).  Which global piece lands in LDS piece p is where the two kinds differ:
+// the XOR swizzles below are applied on the global side.
+
+// ---- operand with contiguous contraction axis: LDS tile [EXT][64], 128 B per row ------------------------
+// piece p = (row, phys) holds contraction chunk c = phys ^ f(row); f makes the 16 lanes of a ds_read_b128
+// phase (16 consecutive rows, one chunk) hit 16 different 16-byte bank groups.
+__device__ __forceinline__ int direct_swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
 template <int EXT, int NT>
 struct DirectOp {
-  static constexpr int CHUNKS = EXT * 8;
-  static constexpr int R = (CHUNKS + NT - 1) / NT;
+  static constexpr int PIECES = EXT * 8;
+  static constexpr int R = PIECES / NT;
   static constexpr int LDS_BYTES = EXT * 128;
-  const char* ptr[R];      // row base (bytes) of the row this thread copies in round i
+  static constexpr int DS_PER_FRAG = 1;
+  static_assert(PIECES % NT == 0, "tile must be a whole number of rounds");
+  const char* ptr[R];      // global address of this thread's piece in round j at contraction 0
   // `row_ptr(row)` returns the global byte address of element (row, k = 0) of the tile's row `row`
   template <typename F>
   __device__ __forceinline__ void init(F row_ptr) {
     const int t = threadIdx.x;
 #pragma unroll
-    for (int i = 0; i < R; ++i) {
-      const int c = t + i * NT;
-      ptr[i] = (c < CHUNKS) ? row_ptr(c >> 3) : nullptr;
+    for (int j = 0; j < R; ++j) {
+      const int p = j * NT + t, row = p >> 3;
+      ptr[j] = row_ptr(row) + (((p & 7) ^ direct_swz(row)) << 4);
     }
   }
-  __device__ __forceinline__ void load(i32x4 (&regs)[R], int k0, int kend) const {
-    const int kk = k0 + (threadIdx.x & 7) * 8;
+  __device__ __forceinline__ void issue(unsigned tile, int k0) const {
+    const unsigned w = tile + wave_uniform_id() * 1024;
 #pragma unroll
-    for (int i = 0; i < R; ++i) {
-      i32x4 v = {0, 0, 0, 0};
-      if (ptr[i] != nullptr && kk < kend) v = *(const i32x4*)(ptr[i] + (int64_t)kk * 2);
-      regs[i] = v;
-    }
+    for (int j = 0; j < R; ++j) load_to_lds16(ptr[j] + (int64_t)k0 * 2, w + j * NT * 16);
   }
-  __device__ __forceinline__ void store(char* tile, const i32x4 (&regs)[R]) const {
+  // Partial last slice: pieces past `kend` are fetched from contraction 0 of the same row (always valid
+  // memory) and overwritten with zeros by the same thread once its loads have landed.
+  __device__ __forceinline__ void issue_tail(unsigned tile, int k0, int kend) const {
+    const unsigned w = tile + wave_uniform_id() * 1024;
     const int t = threadIdx.x;
 #pragma unroll
-    for (int i = 0; i < R; ++i) {
-      const int c = t + i * NT;
-      if (c < CHUNKS) lds_write16(tile + direct_off(c >> 3, c & 7), regs[i]);
+    for (int j = 0; j < R; ++j) {
+      const int p = j * NT + t;
+      const int c = (p & 7) ^ direct_swz(p >> 3);
+      const bool ok = k0 + c * 8 < kend;
+      load_to_lds16(ok ? ptr[j] + (int64_t)k0 * 2 : ptr[j] - (c << 4), w + j * NT * 16);
+    }
+  }
+  __device__ __forceinline__ void zero_tail(char* tile, int k0, int kend) const {
+    const int t = threadIdx.x;
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      const int p = j * NT + t;
+      const int c = (p & 7) ^ direct_swz(p >> 3);
+      if (k0 + c * 8 >= kend) lds_write16(tile + p * 16, i32x4{0, 0, 0, 0});
     }
   }
   // fragment of MFMA operand rows [base, base+32), contraction step ks (16 elements)
   static __device__ __forceinline__ i32x4 frag(const char* tile, int base, int ks) {
     const int l = lane_id();
-    return lds_read16(tile + direct_off(base + (l & 31), 2 * ks + (l >> 5)));
+    const int row = base + (l & 31);
+    return lds_read16(tile + row * 128 + (((2 * ks + (l >> 5)) ^ direct_swz(row)) << 4));
   }
 };
 
-// ---- operand with strided contraction axis: LDS tile [64][EXT] (+pad), read transposed ----------------
+// ---- operand with strided contraction axis: LDS tile [64][EXT], read transposed --------------------------
+// Row kr of the tile is EXT*2 bytes = G granules of 64 B (32 columns).  A ds_read_b64_tr_b16 phase touches
+// one granule column in 4 consecutive rows; storing granule g of row kr at position g ^ (kr & 3) spreads
+// those 4 accesses over all 64 banks.
 template <int EXT, int NT>
 struct TransOp {
-  static constexpr int CPR = EXT / 8;                  // 16-byte chunks per contraction row
-  static constexpr int CHUNKS = 64 * CPR;
-  static constexpr int R = (CHUNKS + NT - 1) / NT;
-  static constexpr int RS = EXT * 2 + kTrPad;          // LDS row stride, bytes
+  static constexpr int CPR = EXT / 8;                  // 16-byte pieces per contraction row
+  static constexpr int PIECES = 64 * CPR;
+  static constexpr int R = PIECES / NT;
+  static constexpr int RS = EXT * 2;                   // LDS row stride, bytes
+  static constexpr int DS_PER_FRAG = 2;
   static constexpr int LDS_BYTES = 64 * RS;
-  const char* base;   // global byte address of (contraction 0, column 0 of the tile)
-  int64_t ld;         // bytes between contraction rows
-  int ncols;          // valid columns of this tile (multiple of 8)
+  static_assert(PIECES % NT == 0 && EXT % 128 == 0, "unsupported transposed tile width");
+  const char* ptr[R];  // global address of this thread's piece in round j at contraction row 0
+  int64_t ld;          // bytes between contraction rows
+  // b: global byte address of (contraction 0, column 0 of the tile); columns >= valid_cols are clamped to
+  // column 0 (they only feed outputs that are never stored)
   __device__ __forceinline__ void init(const char* b, int64_t ld_bytes, int valid_cols) {
-    base = b; ld = ld_bytes; ncols = valid_cols;
-  }
-  __device__ __forceinline__ void load(i32x4 (&regs)[R], int k0, int kend) const {
+    ld = ld_bytes;
     const int t = threadIdx.x;
 #pragma unroll
-    for (int i = 0; i < R; ++i) {
-      const int c = t + i * NT;
-      const int kr = c / CPR, cc = c % CPR;
-      i32x4 v = {0, 0, 0, 0};
-      if (c < CHUNKS && k0 + kr < kend && cc * 8 < ncols)
-        v = *(const i32x4*)(base + (int64_t)(k0 + kr) * ld + cc * 16);
-      regs[i] = v;
+    for (int j = 0; j < R; ++j) {
+      const int p = j * NT + t;
+      const int kr = p / CPR, phys = p % CPR;
+      int cc = ((((phys >> 2) ^ (kr & 3)) << 2) | (phys & 3));      // logical 16-byte piece of the row
+      if (cc * 8 >= valid_cols) cc = 0;
+      ptr[j] = b + (int64_t)kr * ld_bytes + cc * 16;
     }
   }
-  __device__ __forceinline__ void store(char* tile, const i32x4 (&regs)[R]) const {
+  __device__ __forceinline__ void issue(unsigned tile, int k0) const {
+    const unsigned w = tile + wave_uniform_id() * 1024;
+#pragma unroll
+    for (int j = 0; j < R; ++j) load_to_lds16(ptr[j] + (int64_t)k0 * ld, w + j * NT * 16);
+  }
+  // Partial last slice: contraction rows past `kend` are fetched from row 0 of the slice (always valid
+  // memory) and overwritten with zeros by the same thread once its loads have landed.
+  __device__ __forceinline__ void issue_tail(unsigned tile, int k0, int kend) const {
+    const unsigned w = tile + wave_uniform_id() * 1024;
     const int t = threadIdx.x;
 #pragma unroll
-    for (int i = 0; i < R; ++i) {
-      const int c = t + i * NT;
-      if (c < CHUNKS) lds_write16(tile + (c / CPR) * RS + (c % CPR) * 16, regs[i]);
+    for (int j = 0; j < R; ++j) {
+      const int kr = (j * NT + t) / CPR;
+      const bool ok = k0 + kr < kend;
+      load_to_lds16(ptr[j] + (int64_t)(ok ? k0 : k0 - kr) * ld, w + j * NT * 16);
+    }
+  }
+  __device__ __forceinline__ void zero_tail(char* tile, int k0, int kend) const {
+    const int t = threadIdx.x;
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      const int p = j * NT + t;
+      if (k0 + p / CPR >= kend) lds_write16(tile + p * 16, i32x4{0, 0, 0, 0});
     }
   }
   // Each 16-lane block transposes a 4 (contraction) x 16 (columns) patch: lane r of the block points at
@@ -142,9 +199,9 @@ struct TransOp {
   static __device__ __forceinline__ i32x4 frag(const char* tile, int base, int ks) {
     const int l = lane_id();
     const int b = l >> 4, r = l & 15;
-    const int col = base + 16 * (b & 1) + 4 * (r & 3);
     const int kr = ks * 16 + 8 * (b >> 1) + (r >> 2);
-    const char* p = tile + kr * RS + col * 2;
+    const int gran = (base >> 5) ^ (r >> 2);                       // (kr & 3) == r >> 2
+    const char* p = tile + kr * RS + (gran << 6) + (16 * (b & 1) + 4 * (r & 3)) * 2;
     const s16x4 lo = lds_read_tr(p);
     const s16x4 hi = lds_read_tr(p + 4 * RS);
     const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
@@ -162,54 +219,83 @@ struct Tile {
 };
 
 // Main loop shared by both kernels.  acc[i][j] is the 32x32 block (i, j) of this wave's tile.
-// If ROWSUM, rs[i] additionally accumulates, per lane, the sum of the lane's own 8 contraction elements of
+// Full 64-deep slices travel global -> LDS directly (no registers, no ds_write) one slice ahead of the
+// MFMAs; a trailing partial slice is zero-filled in LDS after it has landed.
+// If `rowsum`, rs[i] additionally accumulates, per lane, the sum of the lane's own 8 contraction elements of
 // A-fragment i; adding lanes l and l+32 afterwards gives the sum over the contraction of A row l%32.
 template <typename T, class TL, class AOp, class BOp, bool CAN_ROWSUM>
-__device__ __forceinline__ void mainloop(const AOp& A, const BOp& B, int kbeg, int kend, char* lds, bool rowsum,
+__device__ __forceinline__ void mainloop(const AOp& A, const BOp& B, int klen, char* lds, bool rowsum,
                                          f32x16 (&acc)[TL::FM][TL::FN], float (&rs)[TL::FM]) {
   constexpr int STAGE = AOp::LDS_BYTES + BOp::LDS_BYTES;
   const int wave = threadIdx.x >> 6;
   const int wm = wave / TL::WN, wn = wave % TL::WN;
-  const int nk = (kend - kbeg + BK - 1) / BK;
-  i32x4 ra[AOp::R], rb[BOp::R];
-  if (nk > 0) {
-    A.load(ra, kbeg, kend);
-    B.load(rb, kbeg, kend);
-    A.store(lds, ra);
-    B.store(lds + AOp::LDS_BYTES, rb);
+  const int nfull = klen / BK;
+  const bool tail = (klen % BK) != 0;
+  const int nk = nfull + (tail ? 1 : 0);
+  const unsigned lds_u = lds_address(lds);
+  if (nfull > 0) {
+    A.issue(lds_u, 0);
+    B.issue(lds_u + AOp::LDS_BYTES, 0);
+  } else if (tail) {
+    A.issue_tail(lds_u, 0, klen);
+    B.issue_tail(lds_u + AOp::LDS_BYTES, 0, klen);
   }
-  __syncthreads();
   for (int kt = 0; kt < nk; ++kt) {
     char* cur = lds + (kt & 1) * STAGE;
-    char* nxt = lds + ((kt + 1) & 1) * STAGE;
-    const bool more = kt + 1 < nk;
-    if (more) {
-      A.load(ra, kbeg + (kt + 1) * BK, kend);
-      B.load(rb, kbeg + (kt + 1) * BK, kend);
+    const unsigned nxt = lds_u + ((kt + 1) & 1) * STAGE;
+    __builtin_amdgcn_s_waitcnt(0);   // this thread's direct loads of slice kt have landed in LDS
+    if (tail && kt == nfull) {
+      A.zero_tail(cur, kt * BK, klen);
+      B.zero_tail(cur + AOp::LDS_BYTES, kt * BK, klen);
+    }
+    __syncthreads();                 // ... everyone's have, and everyone is done reading `nxt`
+    if (kt + 1 < nfull) {
+      A.issue(nxt, (kt + 1) * BK);
+      B.issue(nxt + AOp::LDS_BYTES, (kt + 1) * BK);
+    } else if (tail && kt + 1 == nfull) {
+      A.issue_tail(nxt, (kt + 1) * BK, klen);
+      B.issue_tail(nxt + AOp::LDS_BYTES, (kt + 1) * BK, klen);
     }
     const char* ta = cur;
     const char* tb = cur + AOp::LDS_BYTES;
+    i32x4 fa[2][TL::FM], fb[2][TL::FN];
+#pragma unroll
+    for (int i = 0; i < TL::FM; ++i) fa[0][i] = AOp::frag(ta, wm * TL::WTM + i * 32, 0);
+#pragma unroll
+    for (int j = 0; j < TL::FN; ++j) fb[0][j] = BOp::frag(tb, wn * TL::WTN + j * 32, 0);
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
-      i32x4 fa[TL::FM], fb[TL::FN];
+      const int c = ks & 1, n = c ^ 1;
+      if (ks + 1 < BK / 16) {
 #pragma unroll
-      for (int i = 0; i < TL::FM; ++i) fa[i] = AOp::frag(ta, wm * TL::WTM + i * 32, ks);
+        for (int i = 0; i < TL::FM; ++i) fa[n][i] = AOp::frag(ta, wm * TL::WTM + i * 32, ks + 1);
 #pragma unroll
-      for (int j = 0; j < TL::FN; ++j) fb[j] = BOp::frag(tb, wn * TL::WTN + j * 32, ks);
+        for (int j = 0; j < TL::FN; ++j) fb[n][j] = BOp::frag(tb, wn * TL::WTN + j * 32, ks + 1);
+      }
 #pragma unroll
       for (int i = 0; i < TL::FM; ++i)
 #pragma unroll
-        for (int j = 0; j < TL::FN; ++j) acc[i][j] = Mfma<T>::run(fa[i], fb[j], acc[i][j]);
+        for (int j = 0; j < TL::FN; ++j) acc[i][j] = Mfma<T>::run(fa[c][i], fb[c][j], acc[i][j]);
       if (CAN_ROWSUM && rowsum) {
 #pragma unroll
-        for (int i = 0; i < TL::FM; ++i) rs[i] += Mfma<T>::sum8(fa[i]);
+        for (int i = 0; i < TL::FM; ++i) rs[i] += Mfma<T>::sum8(fa[c][i]);
       }
+      // Interleave: the LDS reads of step ks+1 are spread between the MFMAs of step ks.
+      if (ks + 1 < BK / 16) {
+#pragma unroll
+        for (int i = 0; i < TL::FM; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x100, AOp::DS_PER_FRAG, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < TL::FN; ++j) {
+          __builtin_amdgcn_sched_group_barrier(0x100, BOp::DS_PER_FRAG, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, TL::FM * TL::FN - TL::FM - TL::FN, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
-    if (more) {
-      A.store(nxt, ra);
-      B.store(nxt + AOp::LDS_BYTES, rb);
-    }
-    __syncthreads();
   }
 }
 
@@ -323,7 +409,7 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
     for (int j = 0; j < TL::FN; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-  mainloop<T, TL, AOp, BOp, false>(A, B, 0, a.K, lds, false, acc, rs);
+  mainloop<T, TL, AOp, BOp, false>(A, B, a.K, lds, false, acc, rs);
 
   const T* bias = a.b ? (const T*)a.b + (int64_t)e * a.sbe : nullptr;
   epilogue<T, TL>(acc, (T*)a.Y, sDst, n0, a.N, a.syn, bias, a.sbn);
@@ -419,7 +505,7 @@ __global__ __launch_bounds__(TL::NT) void xty_mfma_kernel(XtYPlan a, Raster rast
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
   }
   const bool want_db = a.Db != nullptr && a.db_from_p && n_tile == 0;
-  mainloop<T, TL, AOp, BOp, true>(A, B, 0, r_hi - r_lo, lds, want_db, acc, rs);
+  mainloop<T, TL, AOp, BOp, true>(A, B, r_hi - r_lo, lds, want_db, acc, rs);
 
   epilogue<T, TL>(acc, (T*)a.OUT, sDst, q0, a.nq, 1, nullptr, 0);
 
