@@ -67,12 +67,22 @@ typedef __attribute__((address_space(1))) const void glb_void_t;
 // Issued as inline assembly on purpose: for the builtin the compiler assumes that every later LDS read
 // may alias the in-flight transfer and waits for it (vmcnt(0)) before the first ds_read, which would
 // serialise the prefetch of slice k+1 with the MFMAs of slice k.  The main loop waits explicitly instead.
-// `lds_addr` is the wave-uniform byte address inside the workgroup's LDS allocation.
-__device__ __forceinline__ void load_to_lds16(const char* src, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+// `lds_addr` is the wave-uniform byte address inside the workgroup's LDS allocation; the global address is
+// a wave-uniform 64-bit base (scalar registers) plus a 32-bit per-lane byte offset.  This addressing form
+// matters: the same load with a full 64-bit address in each lane costs the issuing wave so much issue time
+// that the matrix pipe starves (measured: +50% run time for 8 such loads per 32 MFMAs, against no
+// measurable cost for the scalar-base form).
+__device__ __forceinline__ void load_to_lds16(const char* base_uniform, unsigned off, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                :
-               : "s"(lds_addr), "v"(src)
+               : "s"(lds_addr), "v"(off), "s"(base_uniform)
                : "memory", "m0");
+}
+__device__ __forceinline__ const char* make_uniform(const char* p) {
+  const uint64_t v = (uint64_t)p;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return (const char*)(((uint64_t)hi << 32) | lo);
 }
 
 // Both operand kinds fill a 64-deep LDS tile of EXT*128 bytes in LINEAR order of 16-byte pieces: piece
@@ -92,21 +102,24 @@ struct DirectOp {
   static constexpr int LDS_BYTES = EXT * 128;
   static constexpr int DS_PER_FRAG = 1;
   static_assert(PIECES % NT == 0, "tile must be a whole number of rounds");
-  const char* ptr[R];      // global address of this thread's piece in round j at contraction 0
-  // `row_ptr(row)` returns the global byte address of element (row, k = 0) of the tile's row `row`
+  const char* base;        // wave-uniform global address all rows are relative to
+  unsigned off[R];         // byte offset of this thread's piece in round j at contraction 0
+  // `row_off(row)` returns the byte offset (from `b`) of element (row, k = 0) of the tile's row `row`
   template <typename F>
-  __device__ __forceinline__ void init(F row_ptr) {
+  __device__ __forceinline__ void init(const char* b, F row_off) {
+    base = make_uniform(b);
     const int t = threadIdx.x;
 #pragma unroll
     for (int j = 0; j < R; ++j) {
       const int p = j * NT + t, row = p >> 3;
-      ptr[j] = row_ptr(row) + (((p & 7) ^ direct_swz(row)) << 4);
+      off[j] = (unsigned)row_off(row) + (((p & 7) ^ direct_swz(row)) << 4);
     }
   }
   __device__ __forceinline__ void issue(unsigned tile, int k0) const {
     const unsigned w = tile + wave_uniform_id() * 1024;
+    const char* b = base + (int64_t)k0 * 2;
 #pragma unroll
-    for (int j = 0; j < R; ++j) load_to_lds16(ptr[j] + (int64_t)k0 * 2, w + j * NT * 16);
+    for (int j = 0; j < R; ++j) load_to_lds16(b, off[j], w + j * NT * 16);
   }
   // Partial last slice: pieces past `kend` are fetched from contraction 0 of the same row (always valid
   // memory) and overwritten with zeros by the same thread once its loads have landed.
@@ -118,7 +131,7 @@ struct DirectOp {
       const int p = j * NT + t;
       const int c = (p & 7) ^ direct_swz(p >> 3);
       const bool ok = k0 + c * 8 < kend;
-      load_to_lds16(ok ? ptr[j] + (int64_t)k0 * 2 : ptr[j] - (c << 4), w + j * NT * 16);
+      load_to_lds16(base, ok ? off[j] + (unsigned)k0 * 2 : off[j] - (c << 4), w + j * NT * 16);
     }
   }
   __device__ __forceinline__ void zero_tail(char* tile, int k0, int kend) const {
@@ -151,11 +164,12 @@ struct TransOp {
   static constexpr int DS_PER_FRAG = 2;
   static constexpr int LDS_BYTES = 64 * RS;
   static_assert(PIECES % NT == 0 && EXT % 128 == 0, "unsupported transposed tile width");
-  const char* ptr[R];  // global address of this thread's piece in round j at contraction row 0
+  const char* base;    // wave-uniform global address of (contraction 0, column 0 of the tile)
+  unsigned off[R];     // byte offset of this thread's piece in round j within the first slice
   int64_t ld;          // bytes between contraction rows
-  // b: global byte address of (contraction 0, column 0 of the tile); columns >= valid_cols are clamped to
-  // column 0 (they only feed outputs that are never stored)
+  // columns >= valid_cols are clamped to column 0 (they only feed outputs that are never stored)
   __device__ __forceinline__ void init(const char* b, int64_t ld_bytes, int valid_cols) {
+    base = make_uniform(b);
     ld = ld_bytes;
     const int t = threadIdx.x;
 #pragma unroll
@@ -164,24 +178,26 @@ struct TransOp {
       const int kr = p / CPR, phys = p % CPR;
       int cc = ((((phys >> 2) ^ (kr & 3)) << 2) | (phys & 3));      // logical 16-byte piece of the row
       if (cc * 8 >= valid_cols) cc = 0;
-      ptr[j] = b + (int64_t)kr * ld_bytes + cc * 16;
+      off[j] = (unsigned)(kr * ld_bytes) + cc * 16;
     }
   }
   __device__ __forceinline__ void issue(unsigned tile, int k0) const {
     const unsigned w = tile + wave_uniform_id() * 1024;
+    const char* b = base + (int64_t)k0 * ld;
 #pragma unroll
-    for (int j = 0; j < R; ++j) load_to_lds16(ptr[j] + (int64_t)k0 * ld, w + j * NT * 16);
+    for (int j = 0; j < R; ++j) load_to_lds16(b, off[j], w + j * NT * 16);
   }
   // Partial last slice: contraction rows past `kend` are fetched from row 0 of the slice (always valid
   // memory) and overwritten with zeros by the same thread once its loads have landed.
   __device__ __forceinline__ void issue_tail(unsigned tile, int k0, int kend) const {
     const unsigned w = tile + wave_uniform_id() * 1024;
+    const char* b = base + (int64_t)k0 * ld;
     const int t = threadIdx.x;
 #pragma unroll
     for (int j = 0; j < R; ++j) {
       const int kr = (j * NT + t) / CPR;
       const bool ok = k0 + kr < kend;
-      load_to_lds16(ptr[j] + (int64_t)(ok ? k0 : k0 - kr) * ld, w + j * NT * 16);
+      load_to_lds16(b, ok ? off[j] : off[j] - (unsigned)(kr * ld), w + j * NT * 16);
     }
   }
   __device__ __forceinline__ void zero_tail(char* tile, int k0, int kend) const {
@@ -390,7 +406,7 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
   AOp A;
   const char* Xb = (const char*)a.X;
   const int64_t sxm = a.sxm;
-  A.init([&](int row) { return Xb + (int64_t)sSrc[row] * sxm * 2; });
+  A.init(Xb, [&](int row) { return (int64_t)sSrc[row] * sxm * 2; });
   BOp B;
   const char* Wb = (const char*)a.W + (int64_t)e * a.swe * 2;
   if constexpr (B_TR) {
@@ -398,7 +414,7 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
   } else {
     const int64_t swn = a.swn;
     const int N = a.N;
-    B.init([&](int row) { const int n = n0 + row < N ? n0 + row : N - 1; return Wb + (int64_t)n * swn * 2; });
+    B.init(Wb, [&](int row) { const int n = n0 + row < N ? n0 + row : N - 1; return (int64_t)n * swn * 2; });
   }
 
   f32x16 acc[TL::FM][TL::FN];
