@@ -33,7 +33,8 @@ enum { SMOE_F32 = 0, SMOE_BF16 = 1, SMOE_F16 = 2 };
 enum { SMOE_I64 = 0, SMOE_I32 = 1, SMOE_I16 = 2, SMOE_U8 = 3 };
 
 /* activations of the gated linear unit kernels */
-enum { SMOE_ACT_SILU = 0 };
+/* SILU: h = silu(pre[:, f:2f]) * pre[:, 0:f];  SILU_GATE_FIRST: h = silu(pre[:, 0:f]) * pre[:, f:2f] */
+enum { SMOE_ACT_SILU = 0, SMOE_ACT_SILU_GATE_FIRST = 1 };
 
 /* argument errors */
 enum {
@@ -143,6 +144,7 @@ int smoe_gate_grad(const void* Y, int64_t sym, const void* dOut, int64_t sdm, vo
  * Gated linear unit of GLUMLP in one pass:  h = act(pre[:, f:2f]) * pre[:, 0:f]   (first half linear,
  * second half activated), replacing chunk + activation + multiply of scattermoe/mlp.py:81-87, and its
  * gradient  dpre[:, 0:f] = dh * act(g),  dpre[:, f:2f] = dh * lin * act'(g)  that autograd derives from it.
+ * SMOE_ACT_SILU_GATE_FIRST swaps the roles of the halves (the `act(gate) * up` convention of Hugging Face experts).
  * pre / dpre (rows, 2f) row strides spm / sdpm, h / dh (rows, f) row strides shm / sdhm; `act` = SMOE_ACT_*.
  */
 int smoe_glu_fwd(const void* pre, int64_t spm, void* h, int64_t shm, int64_t rows, int64_t f, int act, int dtype,

@@ -133,7 +133,7 @@ int smoe_glu_fwd(const void* pre, int64_t spm, void* h, int64_t shm, int64_t row
   g_err[0] = 0;
   if (!dtype_ok(dtype)) { set_error("smoe_glu_fwd: unknown dtype %d", dtype); return SMOE_ERR_DTYPE; }
   if (rows < 0 || f < 0) { set_error("smoe_glu_fwd: bad sizes"); return SMOE_ERR_SHAPE; }
-  if (act != SMOE_ACT_SILU) { set_error("smoe_glu_fwd: unknown activation %d", act); return SMOE_ERR_SHAPE; }
+  if (act != SMOE_ACT_SILU && act != SMOE_ACT_SILU_GATE_FIRST) { set_error("smoe_glu_fwd: unknown activation %d", act); return SMOE_ERR_SHAPE; }
   if (f > 0x3fffffffLL) { set_error("smoe_glu_fwd: size beyond int32"); return SMOE_ERR_RANGE; }
   if (rows == 0 || f == 0) return 0;
   if (!pre || !h) { set_error("smoe_glu_fwd: NULL pointer"); return SMOE_ERR_NULL; }
@@ -145,7 +145,7 @@ int smoe_glu_bwd(const void* pre, int64_t spm, const void* dh, int64_t sdhm, voi
   g_err[0] = 0;
   if (!dtype_ok(dtype)) { set_error("smoe_glu_bwd: unknown dtype %d", dtype); return SMOE_ERR_DTYPE; }
   if (rows < 0 || f < 0) { set_error("smoe_glu_bwd: bad sizes"); return SMOE_ERR_SHAPE; }
-  if (act != SMOE_ACT_SILU) { set_error("smoe_glu_bwd: unknown activation %d", act); return SMOE_ERR_SHAPE; }
+  if (act != SMOE_ACT_SILU && act != SMOE_ACT_SILU_GATE_FIRST) { set_error("smoe_glu_bwd: unknown activation %d", act); return SMOE_ERR_SHAPE; }
   if (f > 0x3fffffffLL) { set_error("smoe_glu_bwd: size beyond int32"); return SMOE_ERR_RANGE; }
   if (rows == 0 || f == 0) return 0;
   if (!pre || !dh || !dpre) { set_error("smoe_glu_bwd: NULL pointer"); return SMOE_ERR_NULL; }

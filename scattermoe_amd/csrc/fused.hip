@@ -78,6 +78,8 @@ __global__ __launch_bounds__(256) void gate_grad_kernel(const T* __restrict__ Y,
 
 // ---- gated linear unit -----------------------------------------------------------------------------------
 __device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + __expf(-x)); }
+// act & 1 selects which half of `pre` is the activated (gate) half: 0 = second half (GLUMLP of the reference),
+// 1 = first half (the Hugging Face `act(gate) * up` convention).  The activation itself is SiLU.
 __device__ __forceinline__ float act_f(int act, float g) { (void)act; return g * sigmoidf_(g); }
 __device__ __forceinline__ float act_df(int act, float g) {
   (void)act;
@@ -91,18 +93,19 @@ __global__ __launch_bounds__(256) void glu_fwd_kernel(const T* __restrict__ pre,
   constexpr int W = VEC ? Pack<T>::n : 1;
   const int64_t per_row = f / W;
   const int64_t total = rows * per_row;
+  const bool gf = (act & 1) != 0;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
     const int64_t r = i / per_row, c = (i % per_row) * W;
     if (VEC) {
       typedef Pack<T> P;
-      const P lin = *(const P*)(pre + r * sp + c);
-      const P gat = *(const P*)(pre + r * sp + f + c);
+      const P lin = *(const P*)(pre + r * sp + (gf ? f : 0) + c);
+      const P gat = *(const P*)(pre + r * sp + (gf ? 0 : f) + c);
       P o;
 #pragma unroll
       for (int q = 0; q < P::n; ++q) o.v[q] = from_f32<T>(act_f(act, to_f32(gat.v[q])) * to_f32(lin.v[q]));
       *(P*)(h + r * sh + c) = o;
     } else {
-      h[r * sh + c] = from_f32<T>(act_f(act, to_f32(pre[r * sp + f + c])) * to_f32(pre[r * sp + c]));
+      h[r * sh + c] = from_f32<T>(act_f(act, to_f32(pre[r * sp + (gf ? 0 : f) + c])) * to_f32(pre[r * sp + (gf ? f : 0) + c]));
     }
   }
 }
@@ -114,12 +117,13 @@ __global__ __launch_bounds__(256) void glu_bwd_kernel(const T* __restrict__ pre,
   constexpr int W = VEC ? Pack<T>::n : 1;
   const int64_t per_row = f / W;
   const int64_t total = rows * per_row;
+  const bool gf = (act & 1) != 0;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
     const int64_t r = i / per_row, c = (i % per_row) * W;
     if (VEC) {
       typedef Pack<T> P;
-      const P lin = *(const P*)(pre + r * sp + c);
-      const P gat = *(const P*)(pre + r * sp + f + c);
+      const P lin = *(const P*)(pre + r * sp + (gf ? f : 0) + c);
+      const P gat = *(const P*)(pre + r * sp + (gf ? 0 : f) + c);
       const P d = *(const P*)(dh + r * sdh + c);
       P ol, og;
 #pragma unroll
@@ -128,12 +132,12 @@ __global__ __launch_bounds__(256) void glu_bwd_kernel(const T* __restrict__ pre,
         ol.v[q] = from_f32<T>(dv * act_f(act, g));
         og.v[q] = from_f32<T>(dv * to_f32(lin.v[q]) * act_df(act, g));
       }
-      *(P*)(dpre + r * sdp + c) = ol;
-      *(P*)(dpre + r * sdp + f + c) = og;
+      *(P*)(dpre + r * sdp + (gf ? f : 0) + c) = ol;
+      *(P*)(dpre + r * sdp + (gf ? 0 : f) + c) = og;
     } else {
-      const float g = to_f32(pre[r * sp + f + c]), dv = to_f32(dh[r * sdh + c]);
-      dpre[r * sdp + c] = from_f32<T>(dv * act_f(act, g));
-      dpre[r * sdp + f + c] = from_f32<T>(dv * to_f32(pre[r * sp + c]) * act_df(act, g));
+      const float g = to_f32(pre[r * sp + (gf ? 0 : f) + c]), dv = to_f32(dh[r * sdh + c]);
+      dpre[r * sdp + (gf ? f : 0) + c] = from_f32<T>(dv * act_f(act, g));
+      dpre[r * sdp + (gf ? 0 : f) + c] = from_f32<T>(dv * to_f32(pre[r * sp + (gf ? f : 0) + c]) * act_df(act, g));
     }
   }
 }

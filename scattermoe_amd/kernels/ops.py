@@ -285,7 +285,8 @@ def group_compileable(A: torch.Tensor, K: int, N: int, Y: torch.Tensor, coeff: O
 # ------------------------------------------------------------------------------------------------
 # fused passes around the expert GEMMs
 # ------------------------------------------------------------------------------------------------
-ACT_SILU = 0
+ACT_SILU = 0               # h = silu(second half) * first half   (GLUMLP of the reference)
+ACT_SILU_GATE_FIRST = 1    # h = silu(first half) * second half   (Hugging Face `act(gate) * up`)
 
 
 def _rows_contiguous(t):

@@ -1,1 +1,121 @@
-"""Hugging Face injection (placeholder filled in below)."""
+"""Hugging Face injection: route the expert computation of transformers MoE blocks through the
+scattermoe_amd kernels by replacing their `forward` lazily, on first call.
+
+Counterpart of scattermoe/utils/replace_moe.py of the reference: `replace_function` (:8-17),
+`gpt_oss_forward` (:19-57) and `granite_moe_forward` (:60-95).  The reference patches were written against
+transformers 4.5x; the module layouts changed in 5.x (gpt-oss hands the experts already-selected
+(T, k) weights; GraniteMoeHybridMoE owns a router that returns `(top_k_index, top_k_weights, logits)` and an
+`experts` module with `gate_up_proj (E, 2I, H)` / `down_proj (E, H, I)` and returns a single tensor), so each
+forward below accepts both layouts and keeps the return convention of the layout it finds.
+`experts_forward` is the same computation for every 5.x `*Experts.forward(hidden_states, top_k_index,
+top_k_weights)` module (Mixtral, GraniteMoeHybrid, ...); `patch_experts_class(cls)` installs it.
+"""
+import logging
+
+import torch
+from torch import nn
+from torch.nn import functional as F
+
+from ..kernels import ops
+from ..parallel_experts import flatten_sort_count, parallel_linear
+
+
+def replace_function(cls, fun_name):
+    """Decorator: install `fun` as `cls.fun_name`, announcing the swap when it is first used."""
+    def decorator(fun):
+        def first_call(*args, **kwargs):
+            logging.info("Replacing `%s.%s` with %s:%s", cls.__name__, fun_name,
+                         fun.__code__.co_filename, fun.__name__)
+            setattr(cls, fun_name, fun)
+            return fun(*args, **kwargs)
+        first_call.__wrapped__ = fun
+        setattr(cls, fun_name, first_call)
+        return fun
+    return decorator
+
+
+def _glu(pre, act_fn, gate_first):
+    """act(gate) * linear over the two halves of `pre`; fused kernel when the activation is SiLU."""
+    silu = isinstance(act_fn, nn.SiLU) or act_fn is F.silu or type(act_fn).__name__ in ("SiLUActivation", "SiLU")
+    if silu and pre.dim() == 2:
+        from ..mlp import _FusedGLU
+        return _FusedGLU.apply(pre, ops.ACT_SILU_GATE_FIRST if gate_first else ops.ACT_SILU)
+    a, b = pre.chunk(2, dim=-1)
+    return act_fn(a) * b if gate_first else act_fn(b) * a
+
+
+def experts_forward(self, hidden_states, top_k_index, top_k_weights):
+    """Drop-in for transformers 5.x `*Experts.forward`: gate_up_proj (E, 2I, H), down_proj (E, H, I),
+    `act_fn(gate) * up` with gate = first half; returns (T, H)."""
+    k = top_k_index.shape[-1]
+    eid, idx, off = flatten_sort_count(top_k_index, num_experts=self.num_experts)
+    gate_up = parallel_linear(hidden_states, self.gate_up_proj.transpose(1, 2), k, eid, idx, off,
+                              grouped_in=False, grouped_out=True)
+    h = _glu(gate_up, self.act_fn, gate_first=True)
+    return parallel_linear(h, self.down_proj.transpose(1, 2), 1, eid, idx, off,
+                           grouped_in=True, grouped_out=False, gates=top_k_weights.to(h.dtype))
+
+
+def patch_experts_class(cls):
+    """Install `experts_forward` on a transformers 5.x experts class (lazy, like the built-in patches)."""
+    replace_function(cls=cls, fun_name="forward")(experts_forward)
+    return cls
+
+
+try:
+    from transformers.models.gpt_oss.modeling_gpt_oss import GptOssExperts
+
+    @replace_function(cls=GptOssExperts, fun_name="forward")
+    def gpt_oss_forward(self, hidden_states: torch.Tensor, router_indices=None, routing_weights=None) -> torch.Tensor:
+        lead_shape = hidden_states.shape
+        hidden_states = hidden_states.reshape(-1, self.hidden_size)
+        k = router_indices.shape[-1]
+        router_indices = router_indices.reshape(-1, k)
+        routing_weights = routing_weights.reshape(hidden_states.shape[0], -1)
+        if routing_weights.shape[-1] == self.num_experts and k != self.num_experts:
+            # 4.x layout: dense (T, E) scores, pick the routed ones
+            routing_weights = torch.gather(routing_weights, dim=1, index=router_indices)
+        eid, idx, off = flatten_sort_count(router_indices, num_experts=self.num_experts)
+
+        gate_up = parallel_linear(hidden_states, self.gate_up_proj, k, eid, idx, off,
+                                  expert_biases=self.gate_up_proj_bias, grouped_in=False, grouped_out=True)
+        gate, up = gate_up[..., ::2], gate_up[..., 1::2]
+        gate = gate.clamp(min=None, max=self.limit)
+        up = up.clamp(min=-self.limit, max=self.limit)
+        hidden = (up + 1) * (gate * torch.sigmoid(gate * self.alpha))
+
+        out = parallel_linear(hidden, self.down_proj, 1, eid, idx, off,
+                              expert_biases=self.down_proj_bias, grouped_in=True, grouped_out=False,
+                              gates=routing_weights.to(hidden.dtype))
+        if len(lead_shape) == 3:       # 4.x callers pass (batch, seq, hidden) and expect it back
+            return out.view(lead_shape[0], -1, self.hidden_size)
+        return out
+except Exception:   # transformers missing or without this model: nothing to patch
+    logging.info("Failed to replace GptOssExperts")
+
+
+try:
+    from transformers.models.granitemoehybrid.modeling_granitemoehybrid import GraniteMoeHybridMoE
+
+    @replace_function(cls=GraniteMoeHybridMoE, fun_name="forward")
+    def granite_moe_forward(self, layer_input):
+        bsz, length, emb_size = layer_input.size()
+        tokens = layer_input.reshape(-1, emb_size)
+        if hasattr(self, "input_linear"):
+            # 4.x layout: router.layer + input_linear / output_linear, returns (output, router_logits)
+            router_logits = self.router.layer(tokens)
+            weights = F.softmax(router_logits, dim=1, dtype=torch.float)
+            weights, selected = torch.topk(weights, self.router.top_k, dim=-1)
+            weights = (weights / weights.sum(dim=-1, keepdim=True)).to(tokens.dtype)
+            eid, idx, off = flatten_sort_count(selected, num_experts=self.router.num_experts)
+            pre = parallel_linear(tokens, self.input_linear.weight.transpose(2, 1), self.router.top_k,
+                                  eid, idx, off, grouped_in=False, grouped_out=True)
+            h = _glu(pre, self.activation, gate_first=True)
+            out = parallel_linear(h, self.output_linear.weight.transpose(2, 1), 1, eid, idx, off,
+                                  grouped_in=True, grouped_out=False, gates=weights)
+            return out.view(bsz, length, emb_size), router_logits
+        top_k_index, top_k_weights, _ = self.router(tokens)
+        out = experts_forward(self.experts, tokens, top_k_index, top_k_weights)
+        return out.view(bsz, length, self.input_size)
+except Exception:
+    logging.info("Failed to replace GraniteMoeHybridMoE")

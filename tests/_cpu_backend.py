@@ -42,10 +42,15 @@ class OracleBackend:
     @staticmethod
     def glu_fwd(pre, h, act):
         lin, gate = pre.float().chunk(2, dim=-1)
+        if act & 1:
+            lin, gate = gate, lin
         h.copy_(torch.nn.functional.silu(gate) * lin)
 
     @staticmethod
     def glu_bwd(pre, dh, dpre, act):
         lin, gate = pre.float().chunk(2, dim=-1)
+        if act & 1:
+            lin, gate = gate, lin
         s = torch.sigmoid(gate)
-        dpre.copy_(torch.cat([dh.float() * gate * s, dh.float() * lin * s * (1 + gate * (1 - s))], dim=-1))
+        d_lin, d_gate = dh.float() * gate * s, dh.float() * lin * s * (1 + gate * (1 - s))
+        dpre.copy_(torch.cat([d_gate, d_lin] if act & 1 else [d_lin, d_gate], dim=-1))

@@ -1,0 +1,107 @@
+"""GPU parity of the Hugging Face injection and of the decode regime (BASELINE config 5)."""
+import pytest
+import torch
+
+import oracle
+from scattermoe_amd.kernels import ops
+from scattermoe_amd.kernels.single import single2scatter
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _close(got, want, rtol, atol):
+    got, want = got.detach().float().cpu(), want.detach().float()
+    bound = atol * max(1.0, want.abs().max().item()) + rtol * want.abs()
+    err = (got - want).abs()
+    assert bool((err <= bound).all()), "max err %g" % err.max()
+
+
+@pytest.mark.parametrize("dtype,rtol,atol", [(torch.float32, 1e-4, 1e-5), (torch.bfloat16, 2e-2, 1e-2)])
+def test_gpt_oss_patched_forward_backward(dtype, rtol, atol):
+    transformers = pytest.importorskip("transformers")
+    from transformers import GptOssConfig
+    import transformers.models.gpt_oss.modeling_gpt_oss as M
+    from scattermoe_amd.utils import replace_moe as src
+    T, E, k, d, f = 300, 8, 4, 64, 96
+    g = torch.Generator().manual_seed(0)
+    ref = M.GptOssExperts(GptOssConfig(hidden_size=d, intermediate_size=f, num_local_experts=E, num_experts_per_tok=k))
+    with torch.no_grad():
+        for prm in ref.parameters():
+            prm.copy_((torch.randn(prm.shape, generator=g) * 0.2).to(dtype).float())
+    x = torch.randn(T, d, generator=g).to(dtype)
+    top, index = torch.topk(torch.randn(T, E, generator=g), k)
+    weights = torch.softmax(top, -1).to(dtype)
+
+    xc = x.float().requires_grad_()
+    wc = weights.float().requires_grad_()
+    want = oracle.naive_expert_forward(xc, wc, index, ref.gate_up_proj.transpose(1, 2), ref.down_proj.transpose(1, 2),
+                                       oracle.gpt_oss_glu(ref.alpha, ref.limit), ref.gate_up_proj_bias, ref.down_proj_bias)
+    gw = torch.autograd.grad(want, [xc, wc, ref.gate_up_proj, ref.down_proj, ref.gate_up_proj_bias, ref.down_proj_bias],
+                             torch.ones_like(want))
+
+    mod = M.GptOssExperts(GptOssConfig(hidden_size=d, intermediate_size=f, num_local_experts=E, num_experts_per_tok=k))
+    mod.load_state_dict(ref.state_dict())
+    mod = mod.to(DEV).to(dtype)
+    xg = x.to(DEV).requires_grad_()
+    wg = weights.to(DEV).requires_grad_()
+    got = src.gpt_oss_forward(mod, xg, index.to(DEV), wg)
+    gg = torch.autograd.grad(got, [xg, wg, mod.gate_up_proj, mod.down_proj, mod.gate_up_proj_bias, mod.down_proj_bias],
+                             torch.ones_like(got))
+    _close(got, want, rtol, atol)
+    for a, b in zip(gg, gw):
+        _close(a, b, rtol, atol)
+
+
+def test_hf_experts_gate_first_glu():
+    from scattermoe_amd.utils import replace_moe as src
+    T, E, k, d, f = 257, 8, 2, 128, 192
+    g = torch.Generator().manual_seed(1)
+
+    class Experts(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.num_experts = E
+            self.gate_up_proj = torch.nn.Parameter(torch.randn(E, 2 * f, d, generator=g) * 0.1)
+            self.down_proj = torch.nn.Parameter(torch.randn(E, d, f, generator=g) * 0.1)
+            self.act_fn = torch.nn.SiLU()
+
+    m = Experts()
+    x = torch.randn(T, d, generator=g)
+    top, index = torch.topk(torch.randn(T, E, generator=g), k)
+    weights = torch.softmax(top, -1)
+    gate, up = m.gate_up_proj.detach().chunk(2, dim=1)
+    want = oracle.naive_expert_forward(x, weights, index, torch.cat([up, gate], 1), m.down_proj.detach(),
+                                       oracle.glu(torch.nn.functional.silu))
+    mg = Experts().to(DEV)
+    mg.load_state_dict(m.state_dict())
+    got = src.experts_forward(mg, x.to(DEV), index.to(DEV), weights.to(DEV))
+    _close(got, want, 1e-4, 1e-5)
+
+
+@pytest.mark.parametrize("T", [1, 8, 64, 256])
+def test_decode_regime_matches_oracle(T):
+    """Mixtral-shaped decode at reduced width: T tokens, uniform random routing, forward only."""
+    E, k, d, f = 8, 2, 512, 1024
+    g = torch.Generator().manual_seed(T)
+    experts = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)])
+    x = torch.randn(T, d, generator=g).bfloat16()
+    W1 = (torch.randn(E, 2 * f, d, generator=g) * 0.05).bfloat16()
+    eid, idx, off = oracle.route_ref(experts, E)
+    want = oracle.scatter2scatter_ref(x.float(), W1.permute(0, 2, 1).float(), eid, idx, k, None, False, True)
+    r = ops.route(experts.to(DEV), E)
+    assert all(torch.equal(a.cpu(), b) for a, b in zip(r, (eid, idx, off)))
+    got = ops.scatter2scatter(x.to(DEV), W1.to(DEV).permute(0, 2, 1), r[0], r[1], k, y_grouped=True, expert_offsets=r[2])
+    _close(got, want, 2e-2, 1e-2)
+
+
+def test_single2scatter_gpu():
+    g = torch.Generator().manual_seed(2)
+    E, K, N, k = 8, 256, 384, 2
+    W = (torch.randn(E, K, N, generator=g) * 0.1).bfloat16()
+    experts = torch.tensor([[5, 2]])
+    for rows in (1, k):
+        x = torch.randn(rows, K, generator=g).bfloat16()
+        want = torch.stack([x[j if rows == k else 0].float() @ W[e].float() for j, e in enumerate(experts[0])])
+        got = single2scatter(x.to(DEV), W.to(DEV), experts.to(DEV))
+        _close(got, want, 2e-2, 1e-2)
