@@ -33,6 +33,9 @@ def parse():
     ap.add_argument("--workload", default="c2")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-tokens", type=int, default=0, help="token count of the CPU sample (default T/16)")
+    ap.add_argument("--profile-kernel", default="",
+                    help="run ONLY one kernel of the workload `steps` times (for rocprofv3 --pmc): "
+                         "l1fwd | l2fwd | l1dx | l2dx | l1dw | l2dw | copy (a 256 MiB device copy of known size)")
     return ap.parse_args()
 
 
@@ -82,6 +85,46 @@ def cpu_baseline(cfg, tokens, torch):
                       % (cfg.name, tokens, cfg.T, dt, os.cpu_count())}
 
 
+def profile_one_kernel(args, cfg, torch, ops):
+    """Launch one kernel of the workload `steps` times on synthetic operands (no timing, no JSON)."""
+    import scattermoe_amd as sm
+    dev, dt = "cuda:0", cfg.dtype
+    L, d, f, E, k = cfg.T * cfg.k, cfg.d, cfg.f, cfg.E, cfg.k
+    n1 = (2 if cfg.glu else 1) * f
+    g = torch.Generator(device=dev).manual_seed(0)
+    experts = torch.topk(torch.randn(cfg.T, E, generator=g, device=dev), k).indices
+    eid, idx, off = sm.flatten_sort_count(experts, E)
+    r = lambda *shape: torch.randn(*shape, generator=g, device=dev).to(dt)
+    which = args.profile_kernel
+    if which == "l1fwd":
+        X, W = r(cfg.T, d), r(E, n1, d) * 0.02
+        fn = lambda: ops.scatter2scatter(X, W.permute(0, 2, 1), eid, idx, k, y_grouped=True, expert_offsets=off)
+    elif which == "l2fwd":
+        H, W = r(L, f), r(E, d, f) * 0.02
+        fn = lambda: ops.scatter2scatter(H, W.permute(0, 2, 1), eid, idx, 1, x_grouped=True, expert_offsets=off)
+    elif which == "l1dx":
+        G, W = r(L, n1), r(E, n1, d) * 0.02
+        fn = lambda: ops.scatter2scatter(G, W, eid, idx, 1, x_grouped=True, expert_offsets=off)
+    elif which == "l2dx":
+        G, W = r(L, d), r(E, d, f) * 0.02
+        fn = lambda: ops.scatter2scatter(G, W, eid, idx, 1, x_grouped=True, y_grouped=True, expert_offsets=off)
+    elif which == "l1dw":
+        G, X = r(L, n1), r(L, d)
+        fn = lambda: ops.group_bwd_W(G, X, off, E)
+    elif which == "l2dw":
+        G, H = r(L, d), r(L, f)
+        fn = lambda: ops.group_bwd_W(G, H, off, E)
+    elif which == "copy":
+        A = torch.empty(1 << 28, device=dev, dtype=torch.uint8)
+        B = torch.empty_like(A)
+        fn = lambda: B.copy_(A)
+    else:
+        raise SystemExit("unknown --profile-kernel " + which)
+    for _ in range(max(1, args.steps)):
+        fn()
+    torch.cuda.synchronize()
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -103,6 +146,9 @@ def main():
     cfg = CONFIGS[args.workload]
     dev = torch.device("cuda:0")
     dtype = cfg.dtype
+    if args.profile_kernel:
+        profile_one_kernel(args, cfg, torch, ops)
+        return
 
     # synthetic inputs, generated on the device with a fixed seed; resident before timing starts
     g = torch.Generator(device=dev).manual_seed(0)

@@ -453,6 +453,7 @@ static int dispatch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
 }
 
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+static bool fits_u32(int64_t bytes) { return bytes >= 0 && bytes < (int64_t)0xfff00000LL; }
 
 bool try_s2s_mfma(const S2SArgs& a, int dtype, hipStream_t st, int& rc) {
   if (dtype != SMOE_BF16 && dtype != SMOE_F16) return false;
@@ -464,6 +465,11 @@ bool try_s2s_mfma(const S2SArgs& a, int dtype, hipStream_t st, int& rc) {
   if (a.swk == 1 && a.swn % 8 == 0) b_tr = false;
   else if (a.swn == 1 && a.swk % 8 == 0 && a.N % 8 == 0) b_tr = true;
   else return false;
+  // lane offsets inside the kernel are 32-bit byte offsets from a scalar base (X, and W[e])
+  const int64_t x_rows = a.x_grouped ? a.L : a.L / a.fan_out;
+  if (fits_u32((x_rows - 1) * a.sxm * 2 + (int64_t)a.K * 2) == false) return false;
+  if (b_tr ? !fits_u32(BK * a.swk * 2 + (int64_t)a.N * 2) : !fits_u32((int64_t)(a.N - 1) * a.swn * 2 + (int64_t)a.K * 2))
+    return false;
   rc = dtype == SMOE_BF16 ? dispatch_s2s<bf16_t>(a, b_tr, st) : dispatch_s2s<f16_t>(a, b_tr, st);
   return true;
 }
@@ -591,6 +597,7 @@ bool try_xty_mfma(const XtYArgs& a, int dtype, hipStream_t st, int& rc) {
   if (a.sdyn != 1 || a.sxk != 1 || a.sdym % 8 != 0 || a.sxm % 8 != 0) return false;
   if (!aligned16(a.DY) || !aligned16(a.X)) return false;
   if (a.sdwk != 1 && a.sdwn != 1) return false;
+  if (!fits_u32(BK * a.sdym * 2 + (int64_t)a.N * 2) || !fits_u32(BK * a.sxm * 2 + (int64_t)a.K * 2)) return false;
   rc = dtype == SMOE_BF16 ? launch_xty<bf16_t>(a, st) : launch_xty<f16_t>(a, st);
   return true;
 }
