@@ -291,7 +291,7 @@ __device__ __forceinline__ void mainloop(const AOp& A, const BOp& B, int klen, c
 #pragma unroll
       for (int i = 0; i < TL::FM; ++i)
 #pragma unroll
-        for (int j = 0; j < TL::FN; ++j) acc[i][j] = Mfma<T>::run(fa[c][i], fb[c][j], acc[i][j]);
+        for (int j = 0; j < TL::FN; ++j) acc[i][j] = Mfma<T>::run(fb[c][j], fa[c][i], acc[i][j]);
       if (CAN_ROWSUM && rowsum) {
 #pragma unroll
         for (int i = 0; i < TL::FM; ++i) rs[i] += Mfma<T>::sum8(fa[c][i]);
@@ -315,49 +315,68 @@ __device__ __forceinline__ void mainloop(const AOp& A, const BOp& B, int klen, c
   }
 }
 
-// Store the wave's accumulators.  dst[m] is the element offset of output row m of the tile (or -1),
-// columns n0 + [0, BN) clipped to ncols; optional bias (already offset to the expert) with stride sb.
+// Store the wave's accumulators.  The MFMAs are issued with the operands swapped (column operand first), so
+// acc[i][j] holds the TRANSPOSE of output block (i, j): a lane owns output row i*32 + lane%32 and, per group
+// g of four registers, the four consecutive columns j*32 + 8*g + 4*(lane/32) + 0..3 - one 8-byte store per
+// group instead of four 2-byte stores.  dst[m] is the element offset of output row m of the tile (or -1),
+// columns n0 + [0, BN) clipped to ncols (contiguous); optional bias (already offset to the expert), stride sb.
 template <typename T, class TL>
 __device__ __forceinline__ void epilogue(const f32x16 (&acc)[TL::FM][TL::FN], T* __restrict__ out,
-                                         const int64_t* dst, int n0, int ncols, int64_t scol,
+                                         const int64_t* dst, int n0, int ncols,
                                          const T* __restrict__ bias, int64_t sb) {
+  typedef T T4 __attribute__((ext_vector_type(4)));
   const int wave = threadIdx.x >> 6, l = lane_id();
   const int wm = wave / TL::WN, wn = wave % TL::WN;
+  const bool base_ok = ((uintptr_t)out & 7) == 0;
 #pragma unroll
-  for (int j = 0; j < TL::FN; ++j) {
-    const int n = n0 + wn * TL::WTN + j * 32 + (l & 31);
-    const bool nok = n < ncols;
-    const float bv = (bias != nullptr && nok) ? to_f32(bias[(int64_t)n * sb]) : 0.0f;
+  for (int i = 0; i < TL::FM; ++i) {
+    const int64_t d = dst[wm * TL::WTM + i * 32 + (l & 31)];
 #pragma unroll
-    for (int i = 0; i < TL::FM; ++i) {
+    for (int j = 0; j < TL::FN; ++j) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = wm * TL::WTM + i * 32 + (r >> 2) * 8 + (l >> 5) * 4 + (r & 3);
-        const int64_t d = dst[m];
-        if (nok && d >= 0) out[d + (int64_t)n * scol] = from_f32<T>(acc[i][j][r] + bv);
+      for (int g = 0; g < 4; ++g) {
+        const int n = n0 + wn * TL::WTN + j * 32 + g * 8 + (l >> 5) * 4;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[e] = acc[i][j][g * 4 + e];
+          if (bias != nullptr && n + e < ncols) v[e] += to_f32(bias[(int64_t)(n + e) * sb]);
+        }
+        if (d < 0) continue;
+        if (base_ok && n + 3 < ncols && ((d + n) & 3) == 0) {
+          T4 p;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) p[e] = from_f32<T>(v[e]);
+          *(T4*)(out + d + n) = p;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < ncols) out[d + n + e] = from_f32<T>(v[e]);
+        }
       }
     }
   }
 }
 
-// XCD-aware tile order.  Workgroup ids are dealt round-robin to the 8 XCDs (private L2 each), so
-// XCD x = id % 8 takes column groups x, x+8, ... (GN adjacent column tiles each) and sweeps all row
-// tiles of a column group before moving on: the B panels of a group stay in that XCD's L2 while the
-// row panels being swept are shared by all XCDs through the memory-side cache.
+// XCD-aware tile order.  Workgroup ids are dealt round-robin to the 8 XCDs (private L2 each), so the 32
+// workgroups an XCD runs side by side are the ids x, x+8, ..., x+248 of one 256-block; they are mapped to
+// one 8 x 4 "super tile" of output tiles.  Per 64-deep slice that group touches 8 row panels + 4 column
+// panels for 32 tiles' worth of operands, i.e. 3/8 of the requests miss the XCD's L2 instead of 9/16 for
+// a 16 x 2 arrangement and 33/64 for 32 x 1 (measured at the Mixtral shape: 13.3 GB fetched from the
+// memory side per launch against 20.5 GB for 16 x 2).  Super tiles are numbered row-super fastest so that
+// the XCDs working at the same time share column panels through the memory-side cache.
 struct Raster {
-  int m_tiles, n_tiles, gn;
-  __host__ int64_t grid() const {
-    const int supers = (n_tiles + 8 * gn - 1) / (8 * gn);
-    return (int64_t)8 * gn * m_tiles * supers;
-  }
+  static constexpr int SM = 8, SN = 4;
+  int m_tiles, n_tiles, m_supers, supers;
+  int64_t grid_size;                       // host side only: number of workgroups (may exceed what a launch takes)
+  __host__ int64_t grid() const { return grid_size; }
   __device__ __forceinline__ bool map(int pid, int& m, int& n) const {
     const int x = pid & 7, i = pid >> 3;
-    const int nl = i % gn;
-    const int rest = i / gn;
-    m = rest % m_tiles;
-    const int sup = rest / m_tiles;
-    n = (sup * 8 + x) * gn + nl;
-    return n < n_tiles;
+    const int s = (i / (SM * SN)) * 8 + x, r = i % (SM * SN);
+    if (s >= supers) return false;
+    m = (s % m_supers) * SM + r % SM;
+    n = (s / m_supers) * SN + r / SM;
+    return m < m_tiles && n < n_tiles;
   }
 };
 
@@ -365,9 +384,10 @@ static Raster make_raster(int64_t m_tiles, int n_tiles) {
   Raster r;
   r.m_tiles = (int)m_tiles;
   r.n_tiles = n_tiles;
-  r.gn = 1;
-  for (int g = 4; g >= 2; g >>= 1)
-    if (n_tiles % (8 * g) == 0) { r.gn = g; break; }
+  r.m_supers = (int)((m_tiles + Raster::SM - 1) / Raster::SM);
+  const int64_t supers = (int64_t)r.m_supers * ((n_tiles + Raster::SN - 1) / Raster::SN);
+  r.grid_size = (supers + 7) / 8 * 8 * Raster::SM * Raster::SN;
+  r.supers = supers > 0x7fffffffLL ? 0x7fffffff : (int)supers;   // such a grid is rejected by the launchers
   return r;
 }
 
@@ -428,7 +448,7 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
   mainloop<T, TL, AOp, BOp, false>(A, B, a.K, lds, false, acc, rs);
 
   const T* bias = a.b ? (const T*)a.b + (int64_t)e * a.sbe : nullptr;
-  epilogue<T, TL>(acc, (T*)a.Y, sDst, n0, a.N, a.syn, bias, a.sbn);
+  epilogue<T, TL>(acc, (T*)a.Y, sDst, n0, a.N, bias, a.sbn);
 }
 
 template <typename T, class TL>
@@ -529,7 +549,7 @@ __global__ __launch_bounds__(TL::NT) void xty_mfma_kernel(XtYPlan a, Raster rast
   const bool want_db = a.Db != nullptr && a.db_from_p && n_tile == 0;
   mainloop<T, TL, AOp, BOp, true>(A, B, r_hi - r_lo, lds, want_db, acc, rs);
 
-  epilogue<T, TL>(acc, (T*)a.OUT, sDst, q0, a.nq, 1, nullptr, 0);
+  epilogue<T, TL>(acc, (T*)a.OUT, sDst, q0, a.nq, nullptr, 0);
 
   if (want_db) {
     // lanes l and l+32 hold the two contraction halves of row l%32; the first wave column writes the sums
