@@ -22,7 +22,9 @@ PEAK_HBM_GBS = 8000.0
 
 # HBM bytes moved per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (KiB per dispatch, scaled by a copy kernel of known size); None until measured for a workload.
-MEASURED_TRAFFIC = {}
+# c2: average of the two launches of the dominant kernel in a step (layer-1 forward 15.90 GB, layer-2
+# forward 7.00 GB; see profiles/s2s_mfma_c2_l1fwd_counters.md for the commands and raw counter values).
+MEASURED_TRAFFIC = {"c2": 11.45e9}
 
 
 def parse():
