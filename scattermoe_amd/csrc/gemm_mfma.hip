@@ -11,6 +11,9 @@
 // Counterparts in the reference: _scatter2scatter + _compute_expert_block
 // (scattermoe/kernels/ops.py:11-42, 50-118) and _groupXtY + _xty_and_bias (ops.py:242-366).
 #include "common.hpp"
+#ifndef SMOE_RING_BELOW
+#define SMOE_RING_BELOW 24
+#endif
 #include <type_traits>
 
 namespace smoe {
@@ -225,9 +228,10 @@ struct TransOp {
   }
 };
 
-template <int BM_, int BN_, int WM_, int WN_>
+template <int BM_, int BN_, int WM_, int WN_, int NS_ = 2>
 struct Tile {
   static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_;
+  static constexpr int NS = NS_;                      // LDS stages (2: double buffer, more: ring)
   static constexpr int NW = WM * WN, NT = NW * 64;
   static constexpr int WTM = BM / WM, WTN = BN / WN;
   static constexpr int FM = WTM / 32, FN = WTN / 32;
@@ -315,6 +319,67 @@ __device__ __forceinline__ void mainloop(const AOp& A, const BOp& B, int klen, c
   }
 }
 
+// Main loop of the small-row (decode) tile class: memory bound, so what matters is bytes in flight.  The
+// slices travel through a ring of NS stages; NS-1 slices are on their way while one is being multiplied.
+template <typename T, class TL, class AOp, class BOp>
+__device__ __forceinline__ void mainloop_ring(const AOp& A, const BOp& B, int klen, char* lds,
+                                              f32x16 (&acc)[TL::FM][TL::FN]) {
+  constexpr int STAGE = AOp::LDS_BYTES + BOp::LDS_BYTES;
+  constexpr int NS = TL::NS;
+  constexpr int LOADS = AOp::R + BOp::R;               // direct loads per thread and slice
+  static_assert((NS - 2) * LOADS <= 63, "vmcnt cannot count that many loads in flight");
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave / TL::WN, wn = wave % TL::WN;
+  const int nfull = klen / BK;
+  const bool tail = (klen % BK) != 0;
+  const int nk = nfull + (tail ? 1 : 0);
+  const unsigned lds_u = lds_address(lds);
+#define SMOE_RING_ISSUE(s, slot)                                              \
+  do {                                                                        \
+    const unsigned dst_ = lds_u + (slot) * STAGE;                             \
+    if ((s) < nfull) {                                                        \
+      A.issue(dst_, (s) * BK);                                                \
+      B.issue(dst_ + AOp::LDS_BYTES, (s) * BK);                               \
+    } else if ((s) < nk) {                                                    \
+      A.issue_tail(dst_, (s) * BK, klen);                                     \
+      B.issue_tail(dst_ + AOp::LDS_BYTES, (s) * BK, klen);                    \
+    }                                                                         \
+  } while (0)
+#pragma unroll
+  for (int s = 0; s < NS - 1; ++s) SMOE_RING_ISSUE(s, s);
+  int slot = 0;                                        // stage of slice kt
+  for (int kt = 0; kt < nk; ++kt) {
+    // slice kt has landed; the NS-2 younger slices may stay in flight (loads complete in issue order).
+    // Near the end fewer are in flight, so wait for everything there.
+    if (kt + NS - 2 < nk) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 2) * LOADS) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    char* cur = lds + slot * STAGE;
+    if (tail && kt == nfull) {
+      A.zero_tail(cur, kt * BK, klen);
+      B.zero_tail(cur + AOp::LDS_BYTES, kt * BK, klen);
+    }
+    __syncthreads();                 // everyone's part of slice kt is there; everyone is done with slice kt-1
+    const int prev = slot == 0 ? NS - 1 : slot - 1;
+    SMOE_RING_ISSUE(kt + NS - 1, prev);
+    i32x4 fa[BK / 16][TL::FM], fb[BK / 16][TL::FN];
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+#pragma unroll
+      for (int i = 0; i < TL::FM; ++i) fa[ks][i] = AOp::frag(cur, wm * TL::WTM + i * 32, ks);
+#pragma unroll
+      for (int j = 0; j < TL::FN; ++j) fb[ks][j] = BOp::frag(cur + AOp::LDS_BYTES, wn * TL::WTN + j * 32, ks);
+    }
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks)
+#pragma unroll
+      for (int i = 0; i < TL::FM; ++i)
+#pragma unroll
+        for (int j = 0; j < TL::FN; ++j) acc[i][j] = Mfma<T>::run(fb[ks][j], fa[ks][i], acc[i][j]);
+    slot = slot + 1 == NS ? 0 : slot + 1;
+  }
+#undef SMOE_RING_ISSUE
+}
+
 // Store the wave's accumulators.  The MFMAs are issued with the operands swapped (column operand first), so
 // acc[i][j] holds the TRANSPOSE of output block (i, j): a lane owns output row i*32 + lane%32 and, per group
 // g of four registers, the four consecutive columns j*32 + 8*g + 4*(lane/32) + 0..3 - one 8-byte store per
@@ -399,7 +464,7 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
   typedef DirectOp<TL::BM, TL::NT> AOp;
   typedef typename std::conditional<B_TR, TransOp<TL::BN, TL::NT>, DirectOp<TL::BN, TL::NT>>::type BOp;
   constexpr int STAGE = AOp::LDS_BYTES + BOp::LDS_BYTES;
-  __shared__ __attribute__((aligned(16))) char lds[2 * STAGE];
+  __shared__ __attribute__((aligned(16))) char lds[TL::NS * STAGE];
   __shared__ int64_t sDst[TL::BM];
   __shared__ int sSrc[TL::BM];
 
@@ -445,7 +510,8 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
     for (int j = 0; j < TL::FN; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-  mainloop<T, TL, AOp, BOp, false>(A, B, a.K, lds, false, acc, rs);
+  if constexpr (TL::NS > 2) mainloop_ring<T, TL, AOp, BOp>(A, B, a.K, lds, acc);
+  else mainloop<T, TL, AOp, BOp, false>(A, B, a.K, lds, false, acc, rs);
 
   const T* bias = a.b ? (const T*)a.b + (int64_t)e * a.sbe : nullptr;
   epilogue<T, TL>(acc, (T*)a.Y, sDst, n0, a.N, bias, a.sbn);
@@ -469,7 +535,8 @@ static int dispatch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
   const int64_t avg = a.L / a.E;
   if (avg >= 192) return launch_s2s<T, Tile<256, 256, 2, 4>>(a, b_tr, st);
   if (avg >= 96) return launch_s2s<T, Tile<128, 256, 2, 4>>(a, b_tr, st);
-  return launch_s2s<T, Tile<64, 256, 2, 4>>(a, b_tr, st);
+  if (avg >= SMOE_RING_BELOW) return launch_s2s<T, Tile<64, 256, 2, 4>>(a, b_tr, st);
+  return launch_s2s<T, Tile<32, 128, 1, 4, 6>>(a, b_tr, st);
 }
 
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }

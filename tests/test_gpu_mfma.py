@@ -37,7 +37,9 @@ SHAPES = [
     (1100, 8, 2, 200, 264),      # 275 rows/expert: ragged row tails, K % 64 != 0, N % 256 != 0
     (520, 8, 2, 320, 1000),      # 130 rows/expert: 128-row tiles
     (130, 8, 3, 448, 72),        # ~49 rows/expert: 64-row tiles, N < one tile
-    (3, 8, 2, 64, 256),          # decode-like: a handful of rows
+    (3, 8, 2, 64, 256),          # decode-like: a handful of rows (ring-buffered 32-row tiles)
+    (40, 8, 2, 200, 264),        # 10 rows/expert: 32-row tiles with contraction and column tails
+    (9, 4, 2, 1096, 136),        # 32-row tiles, contraction longer than the ring (17 full slices + tail)
     (2048, 32, 4, 192, 328),     # E = 32 with skew: tiny and empty experts
 ]
 
