@@ -14,6 +14,12 @@
 #ifndef SMOE_RING_BELOW
 #define SMOE_RING_BELOW 24
 #endif
+#ifndef SMOE_GM
+#define SMOE_GM 4
+#endif
+#ifndef SMOE_GMX
+#define SMOE_GMX 1000000
+#endif
 #include <type_traits>
 
 namespace smoe {
@@ -432,25 +438,34 @@ __device__ __forceinline__ void epilogue(const f32x16 (&acc)[TL::FM][TL::FN], T*
 // the XCDs working at the same time share column panels through the memory-side cache.
 struct Raster {
   static constexpr int SM = 8, SN = 4;
-  int m_tiles, n_tiles, m_supers, supers;
+  int m_tiles, n_tiles, m_supers, n_supers, supers, gm;
   int64_t grid_size;                       // host side only: number of workgroups (may exceed what a launch takes)
   __host__ int64_t grid() const { return grid_size; }
   __device__ __forceinline__ bool map(int pid, int& m, int& n) const {
     const int x = pid & 7, i = pid >> 3;
     const int s = (i / (SM * SN)) * 8 + x, r = i % (SM * SN);
     if (s >= supers) return false;
-    m = (s % m_supers) * SM + r % SM;
-    n = (s / m_supers) * SN + r / SM;
+    // bands of `gm` row-supers; inside a band column-super major, row-super fastest
+    const int band = s / (gm * n_supers);
+    const int rem = s - band * gm * n_supers;
+    const int g = min(gm, m_supers - band * gm);
+    m = (band * gm + rem % g) * SM + r % SM;
+    n = (rem / g) * SN + r / SM;
     return m < m_tiles && n < n_tiles;
   }
 };
 
-static Raster make_raster(int64_t m_tiles, int n_tiles) {
+// `gm`: row-supers per band.  A band's row panels (gm * 8 tiles) are reused by every column-super while the
+// column panels stream past once, so the band should be small enough for its row panels to stay in the
+// memory-side cache and large enough to keep all XCDs inside one band.
+static Raster make_raster(int64_t m_tiles, int n_tiles, int gm) {
   Raster r;
   r.m_tiles = (int)m_tiles;
   r.n_tiles = n_tiles;
   r.m_supers = (int)((m_tiles + Raster::SM - 1) / Raster::SM);
-  const int64_t supers = (int64_t)r.m_supers * ((n_tiles + Raster::SN - 1) / Raster::SN);
+  r.n_supers = (n_tiles + Raster::SN - 1) / Raster::SN;
+  r.gm = gm < 1 ? 1 : (gm > r.m_supers ? r.m_supers : gm);
+  const int64_t supers = (int64_t)r.m_supers * r.n_supers;
   r.grid_size = (supers + 7) / 8 * 8 * Raster::SM * Raster::SN;
   r.supers = supers > 0x7fffffffLL ? 0x7fffffff : (int)supers;   // such a grid is rejected by the launchers
   return r;
@@ -520,7 +535,7 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
 template <typename T, class TL>
 static int launch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
   const int n_tiles = (a.N + TL::BN - 1) / TL::BN;
-  const Raster r = make_raster(max_tiles(a.L, a.E, TL::BM), n_tiles);
+  const Raster r = make_raster(max_tiles(a.L, a.E, TL::BM), n_tiles, SMOE_GM);
   const int64_t grid = r.grid();
   if (grid > 0x7fffffffLL) { set_error("smoe_scatter2scatter: grid too large"); return SMOE_ERR_RANGE; }
   if (b_tr)
@@ -665,7 +680,7 @@ static int launch_xty(const XtYArgs& a, hipStream_t st) {
   p.db_from_p = k_contig ? 1 : 0;
   const int p_tiles = (p.np + TL::BM - 1) / TL::BM;
   const int q_tiles = (p.nq + TL::BN - 1) / TL::BN;
-  const Raster r = make_raster((int64_t)a.E * p_tiles, q_tiles);
+  const Raster r = make_raster((int64_t)a.E * p_tiles, q_tiles, SMOE_GMX);
   const int64_t grid = r.grid();
   if (grid > 0x7fffffffLL) { set_error("smoe_groupXtY: grid too large"); return SMOE_ERR_RANGE; }
   hipLaunchKernelGGL((xty_mfma_kernel<T, TL>), dim3((unsigned)grid), dim3(TL::NT), 0, st, p, r, p_tiles);
