@@ -538,10 +538,13 @@ static int launch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
   const Raster r = make_raster(max_tiles(a.L, a.E, TL::BM), n_tiles, SMOE_GM);
   const int64_t grid = r.grid();
   if (grid > 0x7fffffffLL) { set_error("smoe_scatter2scatter: grid too large"); return SMOE_ERR_RANGE; }
-  if (b_tr)
-    hipLaunchKernelGGL((s2s_mfma_kernel<T, TL, true>), dim3((unsigned)grid), dim3(TL::NT), 0, st, a, r);
-  else
-    hipLaunchKernelGGL((s2s_mfma_kernel<T, TL, false>), dim3((unsigned)grid), dim3(TL::NT), 0, st, a, r);
+  if constexpr (TL::BN % 128 == 0) {
+    if (b_tr) {
+      hipLaunchKernelGGL((s2s_mfma_kernel<T, TL, true>), dim3((unsigned)grid), dim3(TL::NT), 0, st, a, r);
+      return launch_status("s2s_mfma_kernel");
+    }
+  }
+  hipLaunchKernelGGL((s2s_mfma_kernel<T, TL, false>), dim3((unsigned)grid), dim3(TL::NT), 0, st, a, r);
   return launch_status("s2s_mfma_kernel");
 }
 
@@ -550,7 +553,12 @@ static int dispatch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
   const int64_t avg = a.L / a.E;
   if (avg >= 192) return launch_s2s<T, Tile<256, 256, 2, 4>>(a, b_tr, st);
   if (avg >= 96) return launch_s2s<T, Tile<128, 256, 2, 4>>(a, b_tr, st);
-  if (avg >= SMOE_RING_BELOW) return launch_s2s<T, Tile<64, 256, 2, 4>>(a, b_tr, st);
+  if (avg >= SMOE_RING_BELOW) return launch_s2s<T, Tile<64, 128, 2, 2, 5>>(a, b_tr, st);
+  // Memory-bound class.  With few output columns the 128-wide tiles do not give every CU a workgroup, and what
+  // counts is bytes in flight across the chip: narrower tiles (K-contiguous weights only) restore the count.
+  const int64_t wgs128 = max_tiles(a.L, a.E, 32) * ((a.N + 127) / 128);
+  if (!b_tr && wgs128 < 96) return launch_s2s<T, Tile<32, 32, 1, 1, 8>>(a, b_tr, st);
+  if (!b_tr && wgs128 < 192) return launch_s2s<T, Tile<32, 64, 1, 2, 6>>(a, b_tr, st);
   return launch_s2s<T, Tile<32, 128, 1, 4, 6>>(a, b_tr, st);
 }
 

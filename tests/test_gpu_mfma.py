@@ -40,6 +40,7 @@ SHAPES = [
     (3, 8, 2, 64, 256),          # decode-like: a handful of rows (ring-buffered 32-row tiles)
     (40, 8, 2, 200, 264),        # 10 rows/expert: 32-row tiles with contraction and column tails
     (9, 4, 2, 1096, 136),        # 32-row tiles, contraction longer than the ring (17 full slices + tail)
+    (40, 8, 2, 200, 1288),       # enough 128-wide tiles to pick the 64-wide ring class for K-contiguous weights
     (2048, 32, 4, 192, 328),     # E = 32 with skew: tiny and empty experts
 ]
 
