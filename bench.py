@@ -59,6 +59,26 @@ class TimedBackend:
         c.record()
         self.records.append((a, c, 2.0 * eid.numel() * X.size(1) * Y.size(1), W.stride(1) == 1))
 
+    def _timed(self, fn, flops, k_contig):
+        if not self.on:
+            return fn()
+        a, c = self.torch.cuda.Event(enable_timing=True), self.torch.cuda.Event(enable_timing=True)
+        a.record()
+        ok = fn()
+        c.record()
+        if ok:
+            self.records.append((a, c, flops, k_contig))
+        return ok
+
+    # the fused GEMM + gated-linear-unit launches are launches of the same kernel (scatter2scatter FLOPs only)
+    def s2s_glu(self, X, W, b, pre, h, eid, idx, off, k, x_grouped, act):
+        return self._timed(lambda: self.inner.s2s_glu(X, W, b, pre, h, eid, idx, off, k, x_grouped, act),
+                           2.0 * eid.numel() * X.size(1) * W.size(2), W.stride(1) == 1)
+
+    def s2s_glu_bwd(self, DY, W, pre, dpre, eid, idx, off, act):
+        return self._timed(lambda: self.inner.s2s_glu_bwd(DY, W, pre, dpre, eid, idx, off, act),
+                           2.0 * eid.numel() * DY.size(1) * W.size(2), W.stride(1) == 1)
+
 
 def cpu_baseline(cfg, tokens, torch):
     """Naive per-expert PyTorch path (oracle), fp32, forward + autograd backward, on `tokens` tokens."""

@@ -42,7 +42,9 @@ enum {
   SMOE_ERR_SHAPE = -2,     /* negative / inconsistent sizes */
   SMOE_ERR_DTYPE = -3,     /* unknown dtype enum */
   SMOE_ERR_WORKSPACE = -4, /* workspace too small */
-  SMOE_ERR_RANGE = -5      /* size beyond what the kernels index with (int32 rows, E limit) */
+  SMOE_ERR_RANGE = -5,     /* size beyond what the kernels index with (int32 rows, E limit) */
+  SMOE_ERR_UNSUPPORTED = -6 /* the fused entry point has no kernel for this dtype / layout / shape; nothing was
+                              launched and the caller runs the unfused sequence instead */
 };
 
 /* ABI version of the loaded library (== SMOE_ABI_VERSION it was built with). */
@@ -151,6 +153,38 @@ int smoe_glu_fwd(const void* pre, int64_t spm, void* h, int64_t shm, int64_t row
                  void* stream);
 int smoe_glu_bwd(const void* pre, int64_t spm, const void* dh, int64_t sdhm, void* dpre, int64_t sdpm, int64_t rows,
                  int64_t f, int act, int dtype, void* stream);
+
+/*
+ * Layer 1 of GLUMLP and its gated linear unit in one launch (scattermoe/mlp.py:74-87: the
+ * `self.experts(..., grouped_out=True)` scatter2scatter followed by chunk / activation / multiply):
+ *   pre[n, :] = X[src(n), :] @ W[e(n)] (+ b[e(n)])     (L, 2F), rows in expert-sorted order
+ *   H[n, :]   = act(pre[n, F:2F]) * pre[n, 0:F]        (L, F)   (halves swapped for SMOE_ACT_SILU_GATE_FIRST)
+ * W (E,K,2F) any of the two contiguous layouts, b (E,2F) or NULL.  PRE may be NULL (inference: the
+ * pre-activation is not stored).  H is computed from the pre-activation rounded to `dtype`, i.e. PRE is
+ * bit-identical to smoe_scatter2scatter and H equals smoe_glu_fwd of it up to one unit in the last place on
+ * rare rounding ties of the exponential.  bf16 / fp16 only; returns
+ * SMOE_ERR_UNSUPPORTED (nothing launched) where the matrix-core path does not apply.
+ */
+int smoe_scatter2scatter_glu(const void* X, int64_t sxm, int64_t sxk,
+                             const void* W, int64_t swe, int64_t swk, int64_t swn,
+                             const void* b, int64_t sbe, int64_t sbn,
+                             void* PRE, int64_t spm, void* H, int64_t shm,
+                             const int64_t* eid, const int64_t* idx, const int64_t* off,
+                             int64_t L, int64_t K, int64_t F, int E, int fan_out, int x_grouped,
+                             int act, int dtype, void* stream);
+
+/*
+ * Backward counterpart: the input gradient of layer 2 (scattermoe/parallel_experts.py:108-123, the
+ * scatter2scatter on the transposed weights with grouped rows in and out) fused with the gradient of the gated
+ * linear unit:   dH = DY @ W[e]  (L, F), never stored;   DPRE (L, 2F) from dH and the saved PRE as smoe_glu_bwd.
+ * DY (L,K) grouped rows, W (E,K,F), PRE / DPRE (L,2F) with row strides spm / sdpm.  dH is rounded to `dtype`
+ * first, so the result equals smoe_scatter2scatter + smoe_glu_bwd up to one unit in the last place.  Returns SMOE_ERR_UNSUPPORTED where the matrix-core path does not apply.
+ */
+int smoe_scatter2scatter_glu_bwd(const void* DY, int64_t sdm, int64_t sdk,
+                                 const void* W, int64_t swe, int64_t swk, int64_t swn,
+                                 const void* PRE, int64_t spm, void* DPRE, int64_t sdpm,
+                                 const int64_t* eid, const int64_t* idx, const int64_t* off,
+                                 int64_t L, int64_t K, int64_t F, int E, int act, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

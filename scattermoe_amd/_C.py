@@ -37,7 +37,13 @@ _SIGNATURES = {
     "smoe_gate_grad": (_int, [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _int, _i64, _int, _p]),
     "smoe_glu_fwd": (_int, [_p, _i64, _p, _i64, _i64, _i64, _int, _int, _p]),
     "smoe_glu_bwd": (_int, [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _int, _int, _p]),
+    "smoe_scatter2scatter_glu": (_int, [_p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _i64, _p, _i64, _p, _i64,
+                                        _p, _p, _p, _i64, _i64, _i64, _int, _int, _int, _int, _int, _p]),
+    "smoe_scatter2scatter_glu_bwd": (_int, [_p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _p, _i64,
+                                            _p, _p, _p, _i64, _i64, _i64, _int, _int, _int, _p]),
 }
+
+ERR_UNSUPPORTED = -6
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 

@@ -20,6 +20,50 @@ template <typename T> __device__ __forceinline__ T from_f32(float v) { return (T
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
 
+// ---- gated linear unit math (shared by the stand-alone passes and the fused GEMM epilogues) ----------------
+// Every multiplication / addition below is kept as written (no contraction into FMAs, no reassociation), so
+// that the fused epilogues and the stand-alone passes give the same bits whatever code surrounds them.
+__device__ __forceinline__ float sigmoidf_(float x) {
+#pragma clang fp contract(off) reassociate(off)
+  const float e = __expf(-x);
+  const float d = 1.0f + e;
+  return 1.0f / d;
+}
+// act & 1 selects which half of `pre` is the activated (gate) half: 0 = second half (GLUMLP of the reference),
+// 1 = first half (the Hugging Face `act(gate) * up` convention).  The activation itself is SiLU.
+__device__ __forceinline__ float act_f(int act, float g) {
+#pragma clang fp contract(off) reassociate(off)
+  (void)act;
+  const float s = sigmoidf_(g);
+  return g * s;
+}
+__device__ __forceinline__ float act_df(int act, float g) {
+#pragma clang fp contract(off) reassociate(off)
+  (void)act;
+  const float s = sigmoidf_(g);
+  const float a = 1.0f - s;
+  const float b = g * a;
+  const float c = 1.0f + b;
+  return s * c;
+}
+// hidden value and the two gradients of h = act(gate) * lin
+__device__ __forceinline__ float glu_h(int act, float gat, float lin) {
+#pragma clang fp contract(off) reassociate(off)
+  const float a = act_f(act, gat);
+  return a * lin;
+}
+__device__ __forceinline__ float glu_dlin(int act, float dh, float gat) {
+#pragma clang fp contract(off) reassociate(off)
+  const float a = act_f(act, gat);
+  return dh * a;
+}
+__device__ __forceinline__ float glu_dgat(int act, float dh, float gat, float lin) {
+#pragma clang fp contract(off) reassociate(off)
+  const float t = dh * lin;
+  const float d = act_df(act, gat);
+  return t * d;
+}
+
 // ---- expert-aligned tile lookup -------------------------------------------------------------------
 // Rows are expert-sorted; expert e owns rows [off[e-1], off[e]).  Tiles of height BM never straddle
 // two experts: expert e contributes ceil(count_e / BM) tiles and tiles are numbered expert-major.
@@ -80,6 +124,12 @@ struct S2SArgs {
   const int64_t* eid; const int64_t* idx; const int64_t* off;
   int L, K, N, E, fan_out;
   int x_grouped, y_grouped;
+  // fused gated-linear-unit epilogues (MFMA path only, rows in grouped order):
+  //   glu == 1: W has 2N columns; Y (may be NULL) receives the pre-activation (L, 2N), H the hidden (L, N)
+  //   glu == 2: Y receives d(pre) (L, 2N) computed from the product (= d hidden) and the saved pre-activation AUX
+  int glu = 0, act = 0;
+  const void* aux = nullptr; int64_t saux = 0;
+  void* H = nullptr; int64_t shm = 0;
 };
 
 struct XtYArgs {

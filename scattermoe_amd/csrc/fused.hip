@@ -77,15 +77,7 @@ __global__ __launch_bounds__(256) void gate_grad_kernel(const T* __restrict__ Y,
 }
 
 // ---- gated linear unit -----------------------------------------------------------------------------------
-__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + __expf(-x)); }
-// act & 1 selects which half of `pre` is the activated (gate) half: 0 = second half (GLUMLP of the reference),
-// 1 = first half (the Hugging Face `act(gate) * up` convention).  The activation itself is SiLU.
-__device__ __forceinline__ float act_f(int act, float g) { (void)act; return g * sigmoidf_(g); }
-__device__ __forceinline__ float act_df(int act, float g) {
-  (void)act;
-  const float s = sigmoidf_(g);
-  return s * (1.0f + g * (1.0f - s));
-}
+// sigmoidf_, act_f, act_df: common.hpp
 
 template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void glu_fwd_kernel(const T* __restrict__ pre, int64_t sp, T* __restrict__ h,
@@ -102,10 +94,10 @@ __global__ __launch_bounds__(256) void glu_fwd_kernel(const T* __restrict__ pre,
       const P gat = *(const P*)(pre + r * sp + (gf ? 0 : f) + c);
       P o;
 #pragma unroll
-      for (int q = 0; q < P::n; ++q) o.v[q] = from_f32<T>(act_f(act, to_f32(gat.v[q])) * to_f32(lin.v[q]));
+      for (int q = 0; q < P::n; ++q) o.v[q] = from_f32<T>(glu_h(act, to_f32(gat.v[q]), to_f32(lin.v[q])));
       *(P*)(h + r * sh + c) = o;
     } else {
-      h[r * sh + c] = from_f32<T>(act_f(act, to_f32(pre[r * sp + (gf ? 0 : f) + c])) * to_f32(pre[r * sp + (gf ? f : 0) + c]));
+      h[r * sh + c] = from_f32<T>(glu_h(act, to_f32(pre[r * sp + (gf ? 0 : f) + c]), to_f32(pre[r * sp + (gf ? f : 0) + c])));
     }
   }
 }
@@ -129,15 +121,15 @@ __global__ __launch_bounds__(256) void glu_bwd_kernel(const T* __restrict__ pre,
 #pragma unroll
       for (int q = 0; q < P::n; ++q) {
         const float g = to_f32(gat.v[q]), dv = to_f32(d.v[q]);
-        ol.v[q] = from_f32<T>(dv * act_f(act, g));
-        og.v[q] = from_f32<T>(dv * to_f32(lin.v[q]) * act_df(act, g));
+        ol.v[q] = from_f32<T>(glu_dlin(act, dv, g));
+        og.v[q] = from_f32<T>(glu_dgat(act, dv, g, to_f32(lin.v[q])));
       }
       *(P*)(dpre + r * sdp + (gf ? f : 0) + c) = ol;
       *(P*)(dpre + r * sdp + (gf ? 0 : f) + c) = og;
     } else {
       const float g = to_f32(pre[r * sp + (gf ? 0 : f) + c]), dv = to_f32(dh[r * sdh + c]);
-      dpre[r * sdp + (gf ? f : 0) + c] = from_f32<T>(dv * act_f(act, g));
-      dpre[r * sdp + (gf ? 0 : f) + c] = from_f32<T>(dv * to_f32(pre[r * sp + (gf ? f : 0) + c]) * act_df(act, g));
+      dpre[r * sdp + (gf ? f : 0) + c] = from_f32<T>(glu_dlin(act, dv, g));
+      dpre[r * sdp + (gf ? 0 : f) + c] = from_f32<T>(glu_dgat(act, dv, g, to_f32(pre[r * sp + (gf ? f : 0) + c])));
     }
   }
 }

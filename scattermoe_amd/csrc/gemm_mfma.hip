@@ -178,6 +178,12 @@ struct TransOp {
   int64_t ld;          // bytes between contraction rows
   // columns >= valid_cols are clamped to column 0 (they only feed outputs that are never stored)
   __device__ __forceinline__ void init(const char* b, int64_t ld_bytes, int valid_cols) {
+    init_cols(b, ld_bytes, [&](int tc) { return tc < valid_cols ? tc : 0; });
+  }
+  // `col_of(tc)`: element column (relative to `b`, a multiple of 8, always inside the allocation) that tile
+  // column tc (a multiple of 8) is fetched from
+  template <typename F>
+  __device__ __forceinline__ void init_cols(const char* b, int64_t ld_bytes, F col_of) {
     base = make_uniform(b);
     ld = ld_bytes;
     const int t = threadIdx.x;
@@ -185,9 +191,8 @@ struct TransOp {
     for (int j = 0; j < R; ++j) {
       const int p = j * NT + t;
       const int kr = p / CPR, phys = p % CPR;
-      int cc = ((((phys >> 2) ^ (kr & 3)) << 2) | (phys & 3));      // logical 16-byte piece of the row
-      if (cc * 8 >= valid_cols) cc = 0;
-      off[j] = (unsigned)(kr * ld_bytes) + cc * 16;
+      const int cc = ((((phys >> 2) ^ (kr & 3)) << 2) | (phys & 3));      // logical 16-byte piece of the row
+      off[j] = (unsigned)(kr * ld_bytes) + (unsigned)col_of(cc * 8) * 2;
     }
   }
   __device__ __forceinline__ void issue(unsigned tile, int k0) const {
@@ -429,6 +434,286 @@ __device__ __forceinline__ void epilogue(const f32x16 (&acc)[TL::FM][TL::FN], T*
   }
 }
 
+// ---- epilogues that go through LDS ------------------------------------------------------------------
+// After the main loop the operand buffers are free.  The accumulators (transposed blocks, see `epilogue`) are
+// rounded to the storage type and written to LDS as a row-major BM x BN tile, so that the global traffic of the
+// epilogue can be 16 bytes per lane with a wave covering whole 128-byte lines: 16-byte piece c of row r sits at
+// chunk c ^ (r & (CPR-1)) of the row, which keeps both the 8-byte column-strided writes and the 16-byte
+// row-major reads free of bank conflicts.
+template <class TL>
+__device__ __forceinline__ int staged_addr(int row, int col) {
+  constexpr int CPR = TL::BN / 8;
+  return row * (TL::BN * 2) + ((((col >> 3) ^ row) & (CPR - 1)) << 4) + ((col & 7) << 1);
+}
+
+// `bias_of(tile_col)` returns the value to add to that column (0 without bias).
+template <typename T, class TL, typename BF>
+__device__ __forceinline__ void stage_accumulators(const f32x16 (&acc)[TL::FM][TL::FN], char* lds, BF bias_of) {
+  typedef T T4 __attribute__((ext_vector_type(4)));
+  static_assert(TL::BM * TL::BN * 2 <= TL::NS * (TL::BM + TL::BN) * 128, "staged tile must fit the operand buffers");
+  const int wave = threadIdx.x >> 6, l = lane_id();
+  const int wm = wave / TL::WN, wn = wave % TL::WN;
+  __syncthreads();                                   // every wave is done reading operands
+#pragma unroll
+  for (int j = 0; j < TL::FN; ++j) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int col = wn * TL::WTN + j * 32 + g * 8 + (l >> 5) * 4;
+      float bv[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) bv[e] = bias_of(col + e);
+#pragma unroll
+      for (int i = 0; i < TL::FM; ++i) {
+        const int row = wm * TL::WTM + i * 32 + (l & 31);
+        T4 v;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = from_f32<T>(acc[i][j][g * 4 + e] + bv[e]);
+        *(T4*)(lds + staged_addr<TL>(row, col)) = v;
+      }
+    }
+  }
+  __syncthreads();
+}
+
+// Fused gated-linear-unit epilogues (rows in grouped order: output row = row0 + m).
+// Forward: the column operand of the tile is laid out so that each wave owns WTN/2 "first half" columns
+// (accumulator blocks j < FN/2) and the matching WTN/2 "second half" columns (blocks j + FN/2).  Both are
+// rounded to the storage type first and the hidden value is computed from the rounded values, i.e. the same
+// arithmetic as storing the pre-activation and running the stand-alone pass over it.
+template <typename T, class TL>
+__device__ __forceinline__ void epilogue_glu_fwd(const f32x16 (&acc)[TL::FM][TL::FN], const S2SArgs& a, int row0,
+                                                 int rows, int nh0, const T* __restrict__ bias) {
+  if constexpr (TL::FN % 2 == 0) {
+    typedef T T4 __attribute__((ext_vector_type(4)));
+    constexpr int FH = TL::FN / 2;
+    const int wave = threadIdx.x >> 6, l = lane_id();
+    const int wm = wave / TL::WN, wn = wave % TL::WN;
+    const int F = a.N;
+    const bool gf = (a.act & 1) != 0;
+    T* pre = (T*)a.Y;
+    T* hid = (T*)a.H;
+    const bool vec_ok = (((uintptr_t)pre | (uintptr_t)hid) & 7) == 0 && ((a.sym | a.shm | F) & 3) == 0;
+#pragma unroll
+    for (int i = 0; i < TL::FM; ++i) {
+      const int m = wm * TL::WTM + i * 32 + (l & 31);
+      const int64_t row = row0 + m;
+#pragma unroll
+      for (int j = 0; j < FH; ++j) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int n = nh0 + wn * (TL::WTN / 2) + j * 32 + g * 8 + (l >> 5) * 4;
+          T first[4], second[4], h[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            float v1 = acc[i][j][g * 4 + e], v2 = acc[i][j + FH][g * 4 + e];
+            if (bias != nullptr && n + e < F) {
+              v1 += to_f32(bias[(int64_t)(n + e) * a.sbn]);
+              v2 += to_f32(bias[(int64_t)(F + n + e) * a.sbn]);
+            }
+            first[e] = from_f32<T>(v1);
+            second[e] = from_f32<T>(v2);
+            const float lin = to_f32(gf ? second[e] : first[e]), gat = to_f32(gf ? first[e] : second[e]);
+            h[e] = from_f32<T>(glu_h(a.act, gat, lin));
+          }
+          if (m >= rows) continue;
+          if (vec_ok && n + 3 < F) {
+            if (pre != nullptr) {
+              *(T4*)(pre + row * a.sym + n) = T4{first[0], first[1], first[2], first[3]};
+              *(T4*)(pre + row * a.sym + F + n) = T4{second[0], second[1], second[2], second[3]};
+            }
+            *(T4*)(hid + row * a.shm + n) = T4{h[0], h[1], h[2], h[3]};
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              if (n + e >= F) continue;
+              if (pre != nullptr) {
+                pre[row * a.sym + n + e] = first[e];
+                pre[row * a.sym + F + n + e] = second[e];
+              }
+              hid[row * a.shm + n + e] = h[e];
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+// Backward: the product is d(hidden); it is rounded to the storage type and turned into d(pre-activation)
+// with the saved pre-activation, exactly as the stand-alone pass would do from a stored d(hidden).
+template <typename T, class TL>
+__device__ __forceinline__ void epilogue_glu_bwd(const f32x16 (&acc)[TL::FM][TL::FN], const S2SArgs& a, int row0,
+                                                 int rows, int n0) {
+  typedef T T4 __attribute__((ext_vector_type(4)));
+  const int wave = threadIdx.x >> 6, l = lane_id();
+  const int wm = wave / TL::WN, wn = wave % TL::WN;
+  const int F = a.N;
+  const bool gf = (a.act & 1) != 0;
+  const T* pre = (const T*)a.aux;
+  T* dpre = (T*)a.Y;
+  const bool vec_ok = (((uintptr_t)pre | (uintptr_t)dpre) & 7) == 0 && ((a.sym | a.saux | F) & 3) == 0;
+#pragma unroll
+  for (int i = 0; i < TL::FM; ++i) {
+    const int m = wm * TL::WTM + i * 32 + (l & 31);
+    if (m >= rows) continue;
+    const int64_t row = row0 + m;
+#pragma unroll
+    for (int j = 0; j < TL::FN; ++j) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int n = n0 + wn * TL::WTN + j * 32 + g * 8 + (l >> 5) * 4;
+        if (n >= F) continue;
+        const bool vec = vec_ok && n + 3 < F;
+        T p1[4], p2[4], o1[4], o2[4];
+        if (vec) {
+          const T4 v1 = *(const T4*)(pre + row * a.saux + n), v2 = *(const T4*)(pre + row * a.saux + F + n);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) { p1[e] = v1[e]; p2[e] = v2[e]; }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const bool ok = n + e < F;
+            p1[e] = ok ? pre[row * a.saux + n + e] : from_f32<T>(0.0f);
+            p2[e] = ok ? pre[row * a.saux + F + n + e] : from_f32<T>(0.0f);
+          }
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float dv = to_f32(from_f32<T>(acc[i][j][g * 4 + e]));
+          const float lin = to_f32(gf ? p2[e] : p1[e]), gat = to_f32(gf ? p1[e] : p2[e]);
+          const T d_lin = from_f32<T>(glu_dlin(a.act, dv, gat)), d_gat = from_f32<T>(glu_dgat(a.act, dv, gat, lin));
+          o1[e] = gf ? d_gat : d_lin;
+          o2[e] = gf ? d_lin : d_gat;
+        }
+        if (vec) {
+          *(T4*)(dpre + row * a.sym + n) = T4{o1[0], o1[1], o1[2], o1[3]};
+          *(T4*)(dpre + row * a.sym + F + n) = T4{o2[0], o2[1], o2[2], o2[3]};
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (n + e >= F) continue;
+            dpre[row * a.sym + n + e] = o1[e];
+            dpre[row * a.sym + F + n + e] = o2[e];
+          }
+        }
+      }
+    }
+  }
+}
+
+// Plain store through LDS: dst[m] is the element offset of output row m of the tile (or -1).
+template <typename T, class TL>
+__device__ __forceinline__ void epilogue_staged(const f32x16 (&acc)[TL::FM][TL::FN], T* __restrict__ out,
+                                                const int64_t* dst, int n0, int ncols, const T* __restrict__ bias,
+                                                int64_t sb, char* lds) {
+  typedef T T8 __attribute__((ext_vector_type(8)));
+  constexpr int CPR = TL::BN / 8, PIECES = TL::BM * CPR, PP = PIECES / TL::NT;
+  static_assert(PIECES % TL::NT == 0, "pieces must divide evenly");
+  stage_accumulators<T, TL>(acc, lds, [&](int tc) {
+    return bias != nullptr && n0 + tc < ncols ? to_f32(bias[(int64_t)(n0 + tc) * sb]) : 0.0f;
+  });
+#pragma unroll
+  for (int q = 0; q < PP; ++q) {
+    const int p = q * TL::NT + threadIdx.x;
+    const int row = p / CPR, c = p % CPR, n = n0 + c * 8;
+    const int64_t d = dst[row];
+    if (d >= 0 && n < ncols) *(T8*)(out + d + n) = *(const T8*)(lds + staged_addr<TL>(row, c * 8));
+  }
+}
+
+// Forward GLU through LDS: both halves staged (tile column order: per wave block WTN/2 first-half columns, then
+// the matching second-half columns); per 16-byte piece of hidden columns two LDS reads, three coalesced stores.
+template <typename T, class TL>
+__device__ __forceinline__ void epilogue_glu_fwd_staged(const f32x16 (&acc)[TL::FM][TL::FN], const S2SArgs& a,
+                                                        int row0, int rows, int nh0, const T* __restrict__ bias,
+                                                        char* lds) {
+  if constexpr (TL::FN % 2 == 0) {
+    typedef T T8 __attribute__((ext_vector_type(8)));
+    constexpr int HALF = TL::WTN / 2;
+    constexpr int CPR = TL::BN / 16, PIECES = TL::BM * CPR, PP = PIECES / TL::NT;
+    static_assert(PIECES % TL::NT == 0 && HALF % 8 == 0, "pieces must divide evenly");
+    const int F = a.N;
+    stage_accumulators<T, TL>(acc, lds, [&](int tc) {
+      const int j = tc % TL::WTN;
+      const int hc = nh0 + (tc / TL::WTN) * HALF + j % HALF;
+      return bias != nullptr && hc < F ? to_f32(bias[(int64_t)(hc + (j >= HALF ? F : 0)) * a.sbn]) : 0.0f;
+    });
+    const bool gf = (a.act & 1) != 0;
+    T* pre = (T*)a.Y;
+    T* hid = (T*)a.H;
+#pragma unroll
+    for (int q = 0; q < PP; ++q) {
+      const int p = q * TL::NT + threadIdx.x;
+      const int row = p / CPR, hc = (p % CPR) * 8;            // hidden column inside the tile
+      const int n = nh0 + hc;
+      if (row >= rows || n >= F) continue;
+      const int tc = (hc / HALF) * TL::WTN + hc % HALF;       // tile column of the first-half value
+      const T8 first = *(const T8*)(lds + staged_addr<TL>(row, tc));
+      const T8 second = *(const T8*)(lds + staged_addr<TL>(row, tc + HALF));
+      T8 h;
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        h[e] = from_f32<T>(glu_h(a.act, to_f32(gf ? first[e] : second[e]), to_f32(gf ? second[e] : first[e])));
+      const int64_t r = row0 + row;
+      if (pre != nullptr) {
+        *(T8*)(pre + r * a.sym + n) = first;
+        *(T8*)(pre + r * a.sym + F + n) = second;
+      }
+      *(T8*)(hid + r * a.shm + n) = h;
+    }
+  }
+}
+
+// Backward through LDS: d(hidden) tile staged, then every thread handles 16-byte pieces (8 columns of one row):
+// two coalesced 16-byte loads of the saved pre-activation, two coalesced 16-byte stores of its gradient.
+template <typename T, class TL>
+__device__ __forceinline__ void epilogue_glu_bwd_staged(const f32x16 (&acc)[TL::FM][TL::FN], const S2SArgs& a,
+                                                        int row0, int rows, int n0, char* lds) {
+  typedef T T8 __attribute__((ext_vector_type(8)));
+  constexpr int CPR = TL::BN / 8, PIECES = TL::BM * CPR, PP = PIECES / TL::NT, GRP = PP < 4 ? PP : 4;
+  static_assert(PIECES % TL::NT == 0 && PP % GRP == 0, "pieces must divide evenly");
+  stage_accumulators<T, TL>(acc, lds, [](int) { return 0.0f; });
+  const int F = a.N;
+  const bool gf = (a.act & 1) != 0;
+  const T* pre = (const T*)a.aux;
+  T* dpre = (T*)a.Y;
+#pragma unroll 1
+  for (int q0 = 0; q0 < PP; q0 += GRP) {
+    T8 p1[GRP], p2[GRP], dh[GRP];
+    bool ok[GRP];
+#pragma unroll
+    for (int u = 0; u < GRP; ++u) {
+      const int p = (q0 + u) * TL::NT + threadIdx.x;
+      const int row = p / CPR, c = p % CPR, n = n0 + c * 8;
+      ok[u] = row < rows && n < F;
+      if (ok[u]) {
+        const T* src = pre + (int64_t)(row0 + row) * a.saux + n;
+        p1[u] = *(const T8*)src;
+        p2[u] = *(const T8*)(src + F);
+      }
+      dh[u] = *(const T8*)(lds + staged_addr<TL>(row, c * 8));
+    }
+#pragma unroll
+    for (int u = 0; u < GRP; ++u) {
+      if (!ok[u]) continue;
+      const int p = (q0 + u) * TL::NT + threadIdx.x;
+      const int row = p / CPR, n = n0 + (p % CPR) * 8;
+      T8 o1, o2;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float dv = to_f32(dh[u][e]);
+        const float lin = to_f32(gf ? p2[u][e] : p1[u][e]), gat = to_f32(gf ? p1[u][e] : p2[u][e]);
+        const T d_lin = from_f32<T>(glu_dlin(a.act, dv, gat)), d_gat = from_f32<T>(glu_dgat(a.act, dv, gat, lin));
+        o1[e] = gf ? d_gat : d_lin;
+        o2[e] = gf ? d_lin : d_gat;
+      }
+      T* dst = dpre + (int64_t)(row0 + row) * a.sym + n;
+      *(T8*)dst = o1;
+      *(T8*)(dst + F) = o2;
+    }
+  }
+}
+
 // XCD-aware tile order.  Workgroup ids are dealt round-robin to the 8 XCDs (private L2 each), so the 32
 // workgroups an XCD runs side by side are the ids x, x+8, ..., x+248 of one 256-block; they are mapped to
 // one 8 x 4 "super tile" of output tiles.  Per 64-deep slice that group touches 8 row panels + 4 column
@@ -487,7 +772,8 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
   if (!rast.map(blockIdx.x, m_tile, n_tile)) return;
   int e, row0, rows;
   if (!find_tile<TL::BM>(a.off, a.E, m_tile, e, row0, rows)) return;
-  const int n0 = n_tile * TL::BN;
+  // first output column of the tile; the fused forward GLU tile holds BN/2 columns of each half
+  const int n0 = a.glu == 1 ? n_tile * (TL::BN / 2) : n_tile * TL::BN;
 
   for (int m = threadIdx.x; m < TL::BM; m += TL::NT) {
     const int mm = m < rows ? m : rows - 1;               // tail rows re-read the last valid row
@@ -509,7 +795,21 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
   A.init(Xb, [&](int row) { return (int64_t)sSrc[row] * sxm * 2; });
   BOp B;
   const char* Wb = (const char*)a.W + (int64_t)e * a.swe * 2;
-  if constexpr (B_TR) {
+  if (a.glu == 1) {
+    // tile column tc -> weight column: wave block tc / WTN, first half of the block from [0, F), second from [F, 2F)
+    const int F = a.N;
+    auto wcol = [&](int tc) {
+      const int j = tc % TL::WTN;
+      const int hc = n0 + (tc / TL::WTN) * (TL::WTN / 2) + j % (TL::WTN / 2);
+      return hc < F ? hc + (j >= TL::WTN / 2 ? F : 0) : 0;
+    };
+    if constexpr (B_TR) {
+      B.init_cols(Wb, a.swk * 2, wcol);
+    } else {
+      const int64_t swn = a.swn;
+      B.init(Wb, [&](int row) { return (int64_t)wcol(row) * swn * 2; });
+    }
+  } else if constexpr (B_TR) {
     B.init(Wb + (int64_t)n0 * 2, a.swk * 2, a.N - n0);
   } else {
     const int64_t swn = a.swn;
@@ -529,12 +829,26 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
   else mainloop<T, TL, AOp, BOp, false>(A, B, a.K, lds, false, acc, rs);
 
   const T* bias = a.b ? (const T*)a.b + (int64_t)e * a.sbe : nullptr;
-  epilogue<T, TL>(acc, (T*)a.Y, sDst, n0, a.N, bias, a.sbn);
+  // 16-byte pieces need every row start 16-byte aligned; otherwise the lane-wise epilogues are used
+  if (a.glu == 0) {
+    const bool al16 = (((uintptr_t)a.Y & 15) == 0) && ((a.sym | a.N) & 7) == 0;
+    if (al16) epilogue_staged<T, TL>(acc, (T*)a.Y, sDst, n0, a.N, bias, a.sbn, lds);
+    else epilogue<T, TL>(acc, (T*)a.Y, sDst, n0, a.N, bias, a.sbn);
+  } else if (a.glu == 1) {
+    const bool al16 = ((((uintptr_t)a.Y | (uintptr_t)a.H) & 15) == 0) && ((a.sym | a.shm | a.N) & 7) == 0;
+    if (al16) epilogue_glu_fwd_staged<T, TL>(acc, a, row0, rows, n0, bias, lds);
+    else epilogue_glu_fwd<T, TL>(acc, a, row0, rows, n0, bias);
+  } else {
+    const bool al16 = ((((uintptr_t)a.aux | (uintptr_t)a.Y) & 15) == 0) && ((a.saux | a.sym | a.N) & 7) == 0;
+    if (al16) epilogue_glu_bwd_staged<T, TL>(acc, a, row0, rows, n0, lds);
+    else epilogue_glu_bwd<T, TL>(acc, a, row0, rows, n0);
+  }
 }
 
 template <typename T, class TL>
 static int launch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
-  const int n_tiles = (a.N + TL::BN - 1) / TL::BN;
+  const int bn = a.glu == 1 ? TL::BN / 2 : TL::BN;     // output columns per tile
+  const int n_tiles = (a.N + bn - 1) / bn;
   const Raster r = make_raster(max_tiles(a.L, a.E, TL::BM), n_tiles, SMOE_GM);
   const int64_t grid = r.grid();
   if (grid > 0x7fffffffLL) { set_error("smoe_scatter2scatter: grid too large"); return SMOE_ERR_RANGE; }
@@ -554,6 +868,8 @@ static int dispatch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
   if (avg >= 192) return launch_s2s<T, Tile<256, 256, 2, 4>>(a, b_tr, st);
   if (avg >= 96) return launch_s2s<T, Tile<128, 256, 2, 4>>(a, b_tr, st);
   if (avg >= SMOE_RING_BELOW) return launch_s2s<T, Tile<64, 128, 2, 2, 5>>(a, b_tr, st);
+  // the fused forward GLU epilogue needs two column blocks per wave, which the classes below do not have
+  if (a.glu == 1) return SMOE_ERR_UNSUPPORTED;
   // Memory-bound class.  With few output columns the 128-wide tiles do not give every CU a workgroup, and what
   // counts is bytes in flight across the chip: narrower tiles (K-contiguous weights only) restore the count.
   const int64_t wgs128 = max_tiles(a.L, a.E, 32) * ((a.N + 127) / 128);
@@ -578,7 +894,8 @@ bool try_s2s_mfma(const S2SArgs& a, int dtype, hipStream_t st, int& rc) {
   // lane offsets inside the kernel are 32-bit byte offsets from a scalar base (X, and W[e])
   const int64_t x_rows = a.x_grouped ? a.L : a.L / a.fan_out;
   if (fits_u32((x_rows - 1) * a.sxm * 2 + (int64_t)a.K * 2) == false) return false;
-  if (b_tr ? !fits_u32(BK * a.swk * 2 + (int64_t)a.N * 2) : !fits_u32((int64_t)(a.N - 1) * a.swn * 2 + (int64_t)a.K * 2))
+  const int64_t w_cols = a.glu == 1 ? 2 * (int64_t)a.N : a.N;
+  if (b_tr ? !fits_u32(BK * a.swk * 2 + w_cols * 2) : !fits_u32((w_cols - 1) * a.swn * 2 + (int64_t)a.K * 2))
     return false;
   rc = dtype == SMOE_BF16 ? dispatch_s2s<bf16_t>(a, b_tr, st) : dispatch_s2s<f16_t>(a, b_tr, st);
   return true;
@@ -639,7 +956,10 @@ __global__ __launch_bounds__(TL::NT) void xty_mfma_kernel(XtYPlan a, Raster rast
   const bool want_db = a.Db != nullptr && a.db_from_p && n_tile == 0;
   mainloop<T, TL, AOp, BOp, true>(A, B, r_hi - r_lo, lds, want_db, acc, rs);
 
-  epilogue<T, TL>(acc, (T*)a.OUT, sDst, q0, a.nq, nullptr, 0);
+  if ((((uintptr_t)a.OUT & 15) == 0) && ((a.soe | a.sop | a.nq) & 7) == 0)
+    epilogue_staged<T, TL>(acc, (T*)a.OUT, sDst, q0, a.nq, nullptr, 0, lds);
+  else
+    epilogue<T, TL>(acc, (T*)a.OUT, sDst, q0, a.nq, nullptr, 0);
 
   if (want_db) {
     // lanes l and l+32 hold the two contraction halves of row l%32; the first wave column writes the sums

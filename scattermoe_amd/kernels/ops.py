@@ -130,6 +130,44 @@ class HipBackend:
                                   _C.stream_ptr(pre.device))
         _C.check(rc, "smoe_glu_bwd")
 
+    @staticmethod
+    def s2s_glu(X, W, b, pre, h, eid, idx, off, k, x_grouped, act):
+        """Fused layer-1 GEMM + GLU; False when the library has no fused kernel for this call."""
+        _C.require_gpu(X, "scatter2scatter_glu")
+        lib = _C.load()
+        sbe, sbn = (b.stride(0), b.stride(1)) if b is not None else (0, 0)
+        with torch.cuda.device(X.device):
+            rc = lib.smoe_scatter2scatter_glu(
+                _C.ptr(X), X.stride(0), X.stride(1),
+                _C.ptr(W), W.stride(0), W.stride(1), W.stride(2),
+                _C.ptr(b), sbe, sbn,
+                _C.ptr(pre), pre.stride(0) if pre is not None else 0, _C.ptr(h), h.stride(0),
+                _C.ptr(eid), _C.ptr(idx), _C.ptr(off),
+                eid.numel(), X.size(1), h.size(1), W.size(0), k, int(bool(x_grouped)), act,
+                _C.float_code(X.dtype), _C.stream_ptr(X.device))
+        if rc == _C.ERR_UNSUPPORTED:
+            return False
+        _C.check(rc, "smoe_scatter2scatter_glu")
+        return True
+
+    @staticmethod
+    def s2s_glu_bwd(DY, W, pre, dpre, eid, idx, off, act):
+        """Fused layer-2 input gradient + GLU gradient; False when there is no fused kernel for this call."""
+        _C.require_gpu(DY, "scatter2scatter_glu_bwd")
+        lib = _C.load()
+        with torch.cuda.device(DY.device):
+            rc = lib.smoe_scatter2scatter_glu_bwd(
+                _C.ptr(DY), DY.stride(0), DY.stride(1),
+                _C.ptr(W), W.stride(0), W.stride(1), W.stride(2),
+                _C.ptr(pre), pre.stride(0), _C.ptr(dpre), dpre.stride(0),
+                _C.ptr(eid), _C.ptr(idx), _C.ptr(off),
+                eid.numel(), DY.size(1), W.size(2), W.size(0), act,
+                _C.float_code(DY.dtype), _C.stream_ptr(DY.device))
+        if rc == _C.ERR_UNSUPPORTED:
+            return False
+        _C.check(rc, "smoe_scatter2scatter_glu_bwd")
+        return True
+
 
 _backend = HipBackend()
 
@@ -329,3 +367,47 @@ def glu_bwd(pre, dh, act=ACT_SILU):
     dpre = torch.empty_like(pre)
     _backend.glu_bwd(pre, dh, dpre, act)
     return dpre
+
+
+def scatter2scatter_glu(X, W, sorted_expert_idxs, sorted_scattered_idxs, k, b=None, x_grouped=False,
+                        act=ACT_SILU, expert_offsets=None, need_pre=True):
+    """Layer 1 of a gated MLP with its GLU: returns (pre, h) with rows in expert-sorted order, where
+    pre = scatter2scatter(X, W, ..., y_grouped=True) (L, 2F) and h = glu_fwd(pre) (L, F)
+    (reference mlp.py:74-87).  One fused launch where the library has one, the two calls otherwise (same
+    results up to one unit in the last place of rare elements).  `need_pre=False` (inference) lets the fused launch skip storing `pre`."""
+    L = sorted_expert_idxs.size(0)
+    assert W.dim() == 3 and W.size(1) == X.size(1) and W.size(2) % 2 == 0
+    assert L == (X.size(0) if x_grouped else X.size(0) * k)
+    F = W.size(2) // 2
+    if (X.is_cuda and X.dtype in (torch.bfloat16, torch.float16) and not torch.compiler.is_compiling()
+            and hasattr(_backend, "s2s_glu")):
+        _same_dtype("scatter2scatter_glu", X, W, b)
+        off = expert_offsets if expert_offsets is not None else offsets_from_sorted(sorted_expert_idxs, W.size(0))
+        pre = torch.empty((L, 2 * F), device=X.device, dtype=X.dtype) if need_pre else None
+        h = torch.empty((L, F), device=X.device, dtype=X.dtype)
+        if _backend.s2s_glu(_rows_contiguous(X), W, b, pre, h, _as_i64(sorted_expert_idxs),
+                            _as_i64(sorted_scattered_idxs), _as_i64(off), k, x_grouped, act):
+            return pre, h
+    pre = scatter2scatter(X, W, sorted_expert_idxs, sorted_scattered_idxs, k, b=b, x_grouped=x_grouped,
+                          y_grouped=True, expert_offsets=expert_offsets)
+    return pre, glu_fwd(pre, act)
+
+
+def scatter2scatter_glu_bwd(DY, W, pre, sorted_expert_idxs, sorted_scattered_idxs, act=ACT_SILU,
+                            expert_offsets=None):
+    """d(pre) (L, 2F) from the grouped output gradient DY (L, K) of layer 2, its weights W (E, K, F) and the
+    saved pre-activation: glu_bwd(pre, scatter2scatter(DY, W, grouped in and out)) in one launch where possible."""
+    L = sorted_expert_idxs.size(0)
+    assert DY.size(0) == L and pre.size(0) == L and pre.size(1) == 2 * W.size(2) and W.size(1) == DY.size(1)
+    if (DY.is_cuda and DY.dtype in (torch.bfloat16, torch.float16) and not torch.compiler.is_compiling()
+            and hasattr(_backend, "s2s_glu_bwd")):
+        _same_dtype("scatter2scatter_glu_bwd", DY, W, pre)
+        off = expert_offsets if expert_offsets is not None else offsets_from_sorted(sorted_expert_idxs, W.size(0))
+        pre_c = _rows_contiguous(pre)
+        dpre = torch.empty_like(pre_c)
+        if _backend.s2s_glu_bwd(_rows_contiguous(DY), W, pre_c, dpre, _as_i64(sorted_expert_idxs),
+                                _as_i64(sorted_scattered_idxs), _as_i64(off), act):
+            return dpre
+    dh = scatter2scatter(DY, W, sorted_expert_idxs, sorted_scattered_idxs, 1, x_grouped=True, y_grouped=True,
+                         expert_offsets=expert_offsets)
+    return glu_bwd(pre, dh, act)

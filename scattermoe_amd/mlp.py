@@ -23,6 +23,63 @@ class _FusedGLU(torch.autograd.Function):
         return ops.glu_bwd(pre, dh, ctx.act), None
 
 
+class _GatedMLP(torch.autograd.Function):
+    """The whole gated expert MLP as one autograd node, so that the gated linear unit can ride in the epilogues
+    of the GEMMs around it: forward = layer 1 + GLU (one launch), layer 2, gate-weighted combine; backward =
+    the dataflow of two chained ParallelLinear nodes (reference parallel_experts.py:64-134) with the layer-2
+    input gradient and the GLU gradient in one launch.  Same numerics as the unfused chain (intermediates are rounded to the storage type at the same points)."""
+
+    @staticmethod
+    def forward(ctx, x, w1, b1, w2, b2, gates, eid, idx, off, k, act):
+        # w1 (E, 2F, d), w2 (E, d, F): the ParallelExperts parameters; the kernels take the (E, in, out) views
+        T = x.size(0)
+        need_grad = any(ctx.needs_input_grad[:6])
+        with torch.device(x.device):
+            pre, h = ops.scatter2scatter_glu(x, w1.permute(0, 2, 1), eid, idx, k, b=b1, act=act,
+                                             expert_offsets=off, need_pre=need_grad)
+            expanded = ops.scatter2scatter(h, w2.permute(0, 2, 1), eid, idx, 1, b=b2, x_grouped=True,
+                                           y_grouped=False, expert_offsets=off)
+            kept = expanded.view(T, k, expanded.size(-1))
+            out = ops.combine(kept, gates)
+        if need_grad:
+            ctx.save_for_backward(x, w1, b1, w2, b2, gates, eid, idx, off, pre, h, kept)
+        ctx.k, ctx.act = k, act
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x, w1, b1, w2, b2, gates, eid, idx, off, pre, h, kept = ctx.saved_tensors
+        k, act = ctx.k, ctx.act
+        need_x, need_w1, need_b1, need_w2, need_b2, need_g = ctx.needs_input_grad[:6]
+        need_b1 = need_b1 and b1 is not None
+        need_b2 = need_b2 and b2 is not None
+        E = w1.size(0)
+        if not grad_out.is_contiguous():
+            grad_out = grad_out.contiguous()
+        with torch.device(grad_out.device):
+            d_gates = ops.gate_grad(kept, grad_out) if need_g else None
+            # dY of layer 2 in expert-sorted order, scaled by each row's gate; reuses the expert-output buffer
+            dy = ops.group(grad_out, idx, coeff=gates.reshape(-1).to(grad_out.dtype), fan_out=k,
+                           out=kept.view(-1, kept.size(-1)))
+            d_w2 = d_b2 = None
+            if need_w2 or need_b2:
+                d_w2, d_b2 = ops.group_bwd_W(DY=dy, X=h, expert_offsets=off, E=E, has_bias=b2 is not None)
+                d_w2 = d_w2.permute(0, 2, 1) if need_w2 else None     # back to the parameter layout (E, d, F)
+            d_x = d_w1 = d_b1 = None
+            if need_x or need_w1 or need_b1:
+                dpre = ops.scatter2scatter_glu_bwd(dy, w2, pre, eid, idx, act=act, expert_offsets=off)
+                xg = ops.group(x, idx, fan_out=k)
+                if need_w1 or need_b1:
+                    d_w1, d_b1 = ops.group_bwd_W(DY=dpre, X=xg, expert_offsets=off, E=E, has_bias=b1 is not None)
+                    d_w1 = d_w1.permute(0, 2, 1) if need_w1 else None
+                if need_x:
+                    d_exp = ops.scatter2scatter(dpre, w1, eid, idx, 1, x_grouped=True, y_grouped=False,
+                                                out=xg, expert_offsets=off)
+                    d_x = d_exp if k == 1 else d_exp.view(x.size(0), k, d_exp.size(-1)).sum(-2)
+        return d_x, d_w1, (d_b1 if need_b1 else None), d_w2, (d_b2 if need_b2 else None), d_gates, \
+            None, None, None, None, None
+
+
 class _SparseMLP(nn.Module):
     """Shared body: route once, expert layer 1 (grouped output), activation, expert layer 2 (+gates)."""
 
@@ -78,3 +135,13 @@ class GLUMLP(_SparseMLP):
             return _FusedGLU.apply(pre, ops.ACT_SILU)
         lin, gate = pre.chunk(2, dim=-1)
         return self.activation(gate) * lin
+
+    def forward(self, x: torch.Tensor, expert_p: torch.Tensor, expert_idxs: torch.Tensor):
+        if type(self.activation) is not nn.SiLU or torch.compiler.is_compiling():
+            return super().forward(x, expert_p, expert_idxs)
+        lead = x.shape[:-1]
+        tokens = x.view(-1, x.size(-1))
+        eid, idx, off = flatten_sort_count(expert_idxs, num_experts=self.num_experts)
+        out = _GatedMLP.apply(tokens, self.experts.weight, self.experts.bias, self.output_experts.weight,
+                              self.output_experts.bias, expert_p, eid, idx, off, self.top_k, ops.ACT_SILU)
+        return out.view(*lead, out.size(-1))
