@@ -22,9 +22,10 @@ PEAK_HBM_GBS = 8000.0
 
 # HBM bytes moved per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (KiB per dispatch, scaled by a copy kernel of known size); None until measured for a workload.
-# c2: average of the two launches of the dominant kernel in a step (layer-1 forward 15.90 GB, layer-2
-# forward 7.00 GB; see profiles/s2s_mfma_c2_l1fwd_counters.md for the commands and raw counter values).
-MEASURED_TRAFFIC = {"c2": 11.45e9}
+# c2: average of the two launches of the dominant kernel in a step (layer-1 forward with the gated linear unit
+# in its epilogue 18.19 GB, layer-2 forward 7.03 GB; see profiles/s2s_mfma_c2_l1fwd_counters.md for the commands
+# and raw counter values).
+MEASURED_TRAFFIC = {"c2": 12.61e9}
 
 
 def parse():
@@ -120,7 +121,10 @@ def profile_one_kernel(args, cfg, torch, ops):
     which = args.profile_kernel
     if which == "l1fwd":
         X, W = r(cfg.T, d), r(E, n1, d) * 0.02
-        fn = lambda: ops.scatter2scatter(X, W.permute(0, 2, 1), eid, idx, k, y_grouped=True, expert_offsets=off)
+        if cfg.glu:   # what GLUMLP launches: layer 1 with the gated linear unit in its epilogue
+            fn = lambda: ops.scatter2scatter_glu(X, W.permute(0, 2, 1), eid, idx, k, expert_offsets=off)
+        else:
+            fn = lambda: ops.scatter2scatter(X, W.permute(0, 2, 1), eid, idx, k, y_grouped=True, expert_offsets=off)
     elif which == "l2fwd":
         H, W = r(L, f), r(E, d, f) * 0.02
         fn = lambda: ops.scatter2scatter(H, W.permute(0, 2, 1), eid, idx, 1, x_grouped=True, expert_offsets=off)
@@ -129,7 +133,11 @@ def profile_one_kernel(args, cfg, torch, ops):
         fn = lambda: ops.scatter2scatter(G, W, eid, idx, 1, x_grouped=True, expert_offsets=off)
     elif which == "l2dx":
         G, W = r(L, d), r(E, d, f) * 0.02
-        fn = lambda: ops.scatter2scatter(G, W, eid, idx, 1, x_grouped=True, y_grouped=True, expert_offsets=off)
+        if cfg.glu:   # layer-2 input gradient with the gradient of the gated linear unit in its epilogue
+            P = r(L, n1)
+            fn = lambda: ops.scatter2scatter_glu_bwd(G, W, P, eid, idx, expert_offsets=off)
+        else:
+            fn = lambda: ops.scatter2scatter(G, W, eid, idx, 1, x_grouped=True, y_grouped=True, expert_offsets=off)
     elif which == "l1dw":
         G, X = r(L, n1), r(L, d)
         fn = lambda: ops.group_bwd_W(G, X, off, E)
