@@ -20,6 +20,9 @@
 #ifndef SMOE_GMX
 #define SMOE_GMX 1000000
 #endif
+#ifndef SMOE_OWN
+#define SMOE_OWN 1
+#endif
 #include <type_traits>
 
 namespace smoe {
@@ -112,7 +115,13 @@ struct DirectOp {
   static constexpr int DS_PER_FRAG = 1;
   static_assert(PIECES % NT == 0, "tile must be a whole number of rounds");
   const char* base;        // wave-uniform global address all rows are relative to
-  unsigned off[R];         // byte offset of this thread's piece in round j at contraction 0
+  unsigned off[R];         // byte offset of this thread's piece of load slot j at contraction 0
+  // Load slot j carries round (j + rot) % R of the tile.  The workgroups of a super tile that share a panel use
+  // different rotations, each starting with the rows it is the designated first toucher of: those L2 misses
+  // then start earliest, and the other sharers ask for the same lines later in their own queues, when the
+  // fill is under way or done, instead of piling onto a miss that has only just been issued.
+  int rot = 0;
+  __device__ __forceinline__ int rnd(int j) const { const int r = j + rot; return r >= R ? r - R : r; }
   // `row_off(row)` returns the byte offset (from `b`) of element (row, k = 0) of the tile's row `row`
   template <typename F>
   __device__ __forceinline__ void init(const char* b, F row_off) {
@@ -120,34 +129,35 @@ struct DirectOp {
     const int t = threadIdx.x;
 #pragma unroll
     for (int j = 0; j < R; ++j) {
-      const int p = j * NT + t, row = p >> 3;
+      const int p = rnd(j) * NT + t, row = p >> 3;
       off[j] = (unsigned)row_off(row) + (((p & 7) ^ direct_swz(row)) << 4);
     }
   }
+  __device__ __forceinline__ void issue_one(unsigned tile, int k0, int j) const {
+    load_to_lds16(base + (int64_t)k0 * 2, off[j], tile + wave_uniform_id() * 1024 + rnd(j) * NT * 16);
+  }
   __device__ __forceinline__ void issue(unsigned tile, int k0) const {
-    const unsigned w = tile + wave_uniform_id() * 1024;
-    const char* b = base + (int64_t)k0 * 2;
 #pragma unroll
-    for (int j = 0; j < R; ++j) load_to_lds16(b, off[j], w + j * NT * 16);
+    for (int j = 0; j < R; ++j) issue_one(tile, k0, j);
   }
   // Partial last slice: pieces past `kend` are fetched from contraction 0 of the same row (always valid
   // memory) and overwritten with zeros by the same thread once its loads have landed.
+  __device__ __forceinline__ void issue_tail_one(unsigned tile, int k0, int kend, int j) const {
+    const int p = rnd(j) * NT + threadIdx.x;
+    const int c = (p & 7) ^ direct_swz(p >> 3);
+    const bool ok = k0 + c * 8 < kend;
+    load_to_lds16(base, ok ? off[j] + (unsigned)k0 * 2 : off[j] - (c << 4),
+                  tile + wave_uniform_id() * 1024 + rnd(j) * NT * 16);
+  }
   __device__ __forceinline__ void issue_tail(unsigned tile, int k0, int kend) const {
-    const unsigned w = tile + wave_uniform_id() * 1024;
-    const int t = threadIdx.x;
 #pragma unroll
-    for (int j = 0; j < R; ++j) {
-      const int p = j * NT + t;
-      const int c = (p & 7) ^ direct_swz(p >> 3);
-      const bool ok = k0 + c * 8 < kend;
-      load_to_lds16(base, ok ? off[j] + (unsigned)k0 * 2 : off[j] - (c << 4), w + j * NT * 16);
-    }
+    for (int j = 0; j < R; ++j) issue_tail_one(tile, k0, kend, j);
   }
   __device__ __forceinline__ void zero_tail(char* tile, int k0, int kend) const {
     const int t = threadIdx.x;
 #pragma unroll
     for (int j = 0; j < R; ++j) {
-      const int p = j * NT + t;
+      const int p = rnd(j) * NT + t;
       const int c = (p & 7) ^ direct_swz(p >> 3);
       if (k0 + c * 8 >= kend) lds_write16(tile + p * 16, i32x4{0, 0, 0, 0});
     }
@@ -174,7 +184,9 @@ struct TransOp {
   static constexpr int LDS_BYTES = 64 * RS;
   static_assert(PIECES % NT == 0 && EXT % 128 == 0, "unsupported transposed tile width");
   const char* base;    // wave-uniform global address of (contraction 0, column 0 of the tile)
-  unsigned off[R];     // byte offset of this thread's piece in round j within the first slice
+  unsigned off[R];     // byte offset of this thread's piece of load slot j within the first slice
+  int rot = 0;         // load slot j carries round (j + rot) % R (see DirectOp)
+  __device__ __forceinline__ int rnd(int j) const { const int r = j + rot; return r >= R ? r - R : r; }
   int64_t ld;          // bytes between contraction rows
   // columns >= valid_cols are clamped to column 0 (they only feed outputs that are never stored)
   __device__ __forceinline__ void init(const char* b, int64_t ld_bytes, int valid_cols) {
@@ -189,36 +201,36 @@ struct TransOp {
     const int t = threadIdx.x;
 #pragma unroll
     for (int j = 0; j < R; ++j) {
-      const int p = j * NT + t;
+      const int p = rnd(j) * NT + t;
       const int kr = p / CPR, phys = p % CPR;
       const int cc = ((((phys >> 2) ^ (kr & 3)) << 2) | (phys & 3));      // logical 16-byte piece of the row
       off[j] = (unsigned)(kr * ld_bytes) + (unsigned)col_of(cc * 8) * 2;
     }
   }
+  __device__ __forceinline__ void issue_one(unsigned tile, int k0, int j) const {
+    load_to_lds16(base + (int64_t)k0 * ld, off[j], tile + wave_uniform_id() * 1024 + rnd(j) * NT * 16);
+  }
   __device__ __forceinline__ void issue(unsigned tile, int k0) const {
-    const unsigned w = tile + wave_uniform_id() * 1024;
-    const char* b = base + (int64_t)k0 * ld;
 #pragma unroll
-    for (int j = 0; j < R; ++j) load_to_lds16(b, off[j], w + j * NT * 16);
+    for (int j = 0; j < R; ++j) issue_one(tile, k0, j);
   }
   // Partial last slice: contraction rows past `kend` are fetched from row 0 of the slice (always valid
   // memory) and overwritten with zeros by the same thread once its loads have landed.
+  __device__ __forceinline__ void issue_tail_one(unsigned tile, int k0, int kend, int j) const {
+    const int kr = (rnd(j) * NT + (int)threadIdx.x) / CPR;
+    const bool ok = k0 + kr < kend;
+    load_to_lds16(base + (int64_t)k0 * ld, ok ? off[j] : off[j] - (unsigned)(kr * ld),
+                  tile + wave_uniform_id() * 1024 + rnd(j) * NT * 16);
+  }
   __device__ __forceinline__ void issue_tail(unsigned tile, int k0, int kend) const {
-    const unsigned w = tile + wave_uniform_id() * 1024;
-    const char* b = base + (int64_t)k0 * ld;
-    const int t = threadIdx.x;
 #pragma unroll
-    for (int j = 0; j < R; ++j) {
-      const int kr = (j * NT + t) / CPR;
-      const bool ok = k0 + kr < kend;
-      load_to_lds16(b, ok ? off[j] : off[j] - (unsigned)(kr * ld), w + j * NT * 16);
-    }
+    for (int j = 0; j < R; ++j) issue_tail_one(tile, k0, kend, j);
   }
   __device__ __forceinline__ void zero_tail(char* tile, int k0, int kend) const {
     const int t = threadIdx.x;
 #pragma unroll
     for (int j = 0; j < R; ++j) {
-      const int p = j * NT + t;
+      const int p = rnd(j) * NT + t;
       if (k0 + p / CPR >= kend) lds_write16(tile + p * 16, i32x4{0, 0, 0, 0});
     }
   }
@@ -238,6 +250,27 @@ struct TransOp {
     return __builtin_bit_cast(i32x4, v);
   }
 };
+
+// One slice of both operands, load slots interleaved (A0 B0 A1 B1 ...) so that the rows each operand starts
+// with (see `rot`) are requested first.
+template <class AOp, class BOp>
+__device__ __forceinline__ void issue_slice(const AOp& A, const BOp& B, unsigned dst, int k0) {
+  constexpr int RM = AOp::R > BOp::R ? AOp::R : BOp::R;
+#pragma unroll
+  for (int j = 0; j < RM; ++j) {
+    if (j < AOp::R) A.issue_one(dst, k0, j);
+    if (j < BOp::R) B.issue_one(dst + AOp::LDS_BYTES, k0, j);
+  }
+}
+template <class AOp, class BOp>
+__device__ __forceinline__ void issue_slice_tail(const AOp& A, const BOp& B, unsigned dst, int k0, int kend) {
+  constexpr int RM = AOp::R > BOp::R ? AOp::R : BOp::R;
+#pragma unroll
+  for (int j = 0; j < RM; ++j) {
+    if (j < AOp::R) A.issue_tail_one(dst, k0, kend, j);
+    if (j < BOp::R) B.issue_tail_one(dst + AOp::LDS_BYTES, k0, kend, j);
+  }
+}
 
 template <int BM_, int BN_, int WM_, int WN_, int NS_ = 2>
 struct Tile {
@@ -264,13 +297,8 @@ __device__ __forceinline__ void mainloop(const AOp& A, const BOp& B, int klen, c
   const bool tail = (klen % BK) != 0;
   const int nk = nfull + (tail ? 1 : 0);
   const unsigned lds_u = lds_address(lds);
-  if (nfull > 0) {
-    A.issue(lds_u, 0);
-    B.issue(lds_u + AOp::LDS_BYTES, 0);
-  } else if (tail) {
-    A.issue_tail(lds_u, 0, klen);
-    B.issue_tail(lds_u + AOp::LDS_BYTES, 0, klen);
-  }
+  if (nfull > 0) issue_slice(A, B, lds_u, 0);
+  else if (tail) issue_slice_tail(A, B, lds_u, 0, klen);
   for (int kt = 0; kt < nk; ++kt) {
     char* cur = lds + (kt & 1) * STAGE;
     const unsigned nxt = lds_u + ((kt + 1) & 1) * STAGE;
@@ -280,13 +308,8 @@ __device__ __forceinline__ void mainloop(const AOp& A, const BOp& B, int klen, c
       B.zero_tail(cur + AOp::LDS_BYTES, kt * BK, klen);
     }
     __syncthreads();                 // ... everyone's have, and everyone is done reading `nxt`
-    if (kt + 1 < nfull) {
-      A.issue(nxt, (kt + 1) * BK);
-      B.issue(nxt + AOp::LDS_BYTES, (kt + 1) * BK);
-    } else if (tail && kt + 1 == nfull) {
-      A.issue_tail(nxt, (kt + 1) * BK, klen);
-      B.issue_tail(nxt + AOp::LDS_BYTES, (kt + 1) * BK, klen);
-    }
+    if (kt + 1 < nfull) issue_slice(A, B, nxt, (kt + 1) * BK);
+    else if (tail && kt + 1 == nfull) issue_slice_tail(A, B, nxt, (kt + 1) * BK, klen);
     const char* ta = cur;
     const char* tb = cur + AOp::LDS_BYTES;
     i32x4 fa[2][TL::FM], fb[2][TL::FN];
@@ -348,13 +371,8 @@ __device__ __forceinline__ void mainloop_ring(const AOp& A, const BOp& B, int kl
 #define SMOE_RING_ISSUE(s, slot)                                              \
   do {                                                                        \
     const unsigned dst_ = lds_u + (slot) * STAGE;                             \
-    if ((s) < nfull) {                                                        \
-      A.issue(dst_, (s) * BK);                                                \
-      B.issue(dst_ + AOp::LDS_BYTES, (s) * BK);                               \
-    } else if ((s) < nk) {                                                    \
-      A.issue_tail(dst_, (s) * BK, klen);                                     \
-      B.issue_tail(dst_ + AOp::LDS_BYTES, (s) * BK, klen);                    \
-    }                                                                         \
+    if ((s) < nfull) issue_slice(A, B, dst_, (s) * BK);                       \
+    else if ((s) < nk) issue_slice_tail(A, B, dst_, (s) * BK, klen);          \
   } while (0)
 #pragma unroll
   for (int s = 0; s < NS - 1; ++s) SMOE_RING_ISSUE(s, s);
@@ -726,10 +744,13 @@ struct Raster {
   int m_tiles, n_tiles, m_supers, n_supers, supers, gm;
   int64_t grid_size;                       // host side only: number of workgroups (may exceed what a launch takes)
   __host__ int64_t grid() const { return grid_size; }
-  __device__ __forceinline__ bool map(int pid, int& m, int& n) const {
+  // (ml, nl): position of the tile inside its super tile
+  __device__ __forceinline__ bool map(int pid, int& m, int& n, int& ml, int& nl) const {
     const int x = pid & 7, i = pid >> 3;
     const int s = (i / (SM * SN)) * 8 + x, r = i % (SM * SN);
     if (s >= supers) return false;
+    ml = r % SM;
+    nl = r / SM;
     // bands of `gm` row-supers; inside a band column-super major, row-super fastest
     const int band = s / (gm * n_supers);
     const int rem = s - band * gm * n_supers;
@@ -768,8 +789,8 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
   __shared__ int64_t sDst[TL::BM];
   __shared__ int sSrc[TL::BM];
 
-  int m_tile, n_tile;
-  if (!rast.map(blockIdx.x, m_tile, n_tile)) return;
+  int m_tile, n_tile, m_loc, n_loc;
+  if (!rast.map(blockIdx.x, m_tile, n_tile, m_loc, n_loc)) return;
   int e, row0, rows;
   if (!find_tile<TL::BM>(a.off, a.E, m_tile, e, row0, rows)) return;
   // first output column of the tile; the fused forward GLU tile holds BN/2 columns of each half
@@ -790,10 +811,12 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
   __syncthreads();
 
   AOp A;
+  A.rot = SMOE_OWN ? (n_loc * AOp::R / Raster::SN) % AOp::R : 0;      // the row panel has SN sharers
   const char* Xb = (const char*)a.X;
   const int64_t sxm = a.sxm;
   A.init(Xb, [&](int row) { return (int64_t)sSrc[row] * sxm * 2; });
   BOp B;
+  B.rot = SMOE_OWN ? (m_loc * BOp::R / Raster::SM) % BOp::R : 0;      // the column panel has SM sharers
   const char* Wb = (const char*)a.W + (int64_t)e * a.swe * 2;
   if (a.glu == 1) {
     // tile column tc -> weight column: wave block tc / WTN, first half of the block from [0, F), second from [F, 2F)
@@ -926,8 +949,8 @@ __global__ __launch_bounds__(TL::NT) void xty_mfma_kernel(XtYPlan a, Raster rast
   __shared__ __attribute__((aligned(16))) char lds[2 * STAGE];
   __shared__ int64_t sDst[TL::BM];
 
-  int m_tile, n_tile;
-  if (!rast.map(blockIdx.x, m_tile, n_tile)) return;
+  int m_tile, n_tile, m_loc, n_loc;
+  if (!rast.map(blockIdx.x, m_tile, n_tile, m_loc, n_loc)) return;
   const int e = m_tile / p_tiles;
   const int p0 = (m_tile % p_tiles) * TL::BM;
   const int q0 = n_tile * TL::BN;
@@ -940,7 +963,7 @@ __global__ __launch_bounds__(TL::NT) void xty_mfma_kernel(XtYPlan a, Raster rast
 
   AOp A;
   A.init((const char*)a.P + ((int64_t)r_lo * a.ldp + p0) * 2, a.ldp * 2, a.np - p0);
-  BOp B;
+  BOp B;           // (rotated load order measured 1.5 % slower here, so both operands keep rot = 0)
   B.init((const char*)a.Q + ((int64_t)r_lo * a.ldq + q0) * 2, a.ldq * 2, a.nq - q0);
 
   f32x16 acc[TL::FM][TL::FN];
