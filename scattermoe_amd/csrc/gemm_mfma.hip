@@ -645,7 +645,7 @@ template <typename T, class TL>
 __device__ __forceinline__ void epilogue_glu_fwd_staged(const f32x16 (&acc)[TL::FM][TL::FN], const S2SArgs& a,
                                                         int row0, int rows, int nh0, const T* __restrict__ bias,
                                                         char* lds) {
-  if constexpr (TL::FN % 2 == 0) {
+  {
     typedef T T8 __attribute__((ext_vector_type(8)));
     constexpr int HALF = TL::WTN / 2;
     constexpr int CPR = TL::BN / 16, PIECES = TL::BM * CPR, PP = PIECES / TL::NT;
@@ -891,8 +891,9 @@ static int dispatch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
   if (avg >= 192) return launch_s2s<T, Tile<256, 256, 2, 4>>(a, b_tr, st);
   if (avg >= 96) return launch_s2s<T, Tile<128, 256, 2, 4>>(a, b_tr, st);
   if (avg >= SMOE_RING_BELOW) return launch_s2s<T, Tile<64, 128, 2, 2, 5>>(a, b_tr, st);
-  // the fused forward GLU epilogue needs two column blocks per wave, which the classes below do not have
-  if (a.glu == 1) return SMOE_ERR_UNSUPPORTED;
+  // With one column block per wave the fused forward GLU exists only in its LDS-staged form (16-byte pieces)
+  if (a.glu == 1 && !((((uintptr_t)a.Y | (uintptr_t)a.H) & 15) == 0 && ((a.sym | a.shm | a.N) & 7) == 0))
+    return SMOE_ERR_UNSUPPORTED;
   // Memory-bound class.  With few output columns the 128-wide tiles do not give every CU a workgroup, and what
   // counts is bytes in flight across the chip: narrower tiles (K-contiguous weights only) restore the count.
   const int64_t wgs128 = max_tiles(a.L, a.E, 32) * ((a.N + 127) / 128);
