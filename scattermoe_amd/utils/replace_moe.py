@@ -34,9 +34,26 @@ def replace_function(cls, fun_name):
     return decorator
 
 
+def _is_silu(act_fn):
+    return isinstance(act_fn, nn.SiLU) or act_fn is F.silu or type(act_fn).__name__ in ("SiLUActivation", "SiLU")
+
+
+def _gated_mlp(tokens, gate_up_w, down_w, k, eid, idx, off, weights, act_fn):
+    """Gated expert MLP with `act(gate) * up`, gate = first half of the (E, 2I, H) layer-1 weights.  With SiLU the
+    whole block is one autograd node whose GLU rides in the GEMM epilogues; other activations use three nodes."""
+    if _is_silu(act_fn) and tokens.dim() == 2 and not torch.compiler.is_compiling():
+        from ..mlp import _GatedMLP
+        return _GatedMLP.apply(tokens, gate_up_w, None, down_w, None, weights.to(tokens.dtype), eid, idx, off, k,
+                               ops.ACT_SILU_GATE_FIRST)
+    pre = parallel_linear(tokens, gate_up_w.transpose(1, 2), k, eid, idx, off, grouped_in=False, grouped_out=True)
+    h = _glu(pre, act_fn, gate_first=True)
+    return parallel_linear(h, down_w.transpose(1, 2), 1, eid, idx, off, grouped_in=True, grouped_out=False,
+                           gates=weights.to(h.dtype))
+
+
 def _glu(pre, act_fn, gate_first):
     """act(gate) * linear over the two halves of `pre`; fused kernel when the activation is SiLU."""
-    silu = isinstance(act_fn, nn.SiLU) or act_fn is F.silu or type(act_fn).__name__ in ("SiLUActivation", "SiLU")
+    silu = _is_silu(act_fn)
     if silu and pre.dim() == 2:
         from ..mlp import _FusedGLU
         return _FusedGLU.apply(pre, ops.ACT_SILU_GATE_FIRST if gate_first else ops.ACT_SILU)
@@ -49,11 +66,7 @@ def experts_forward(self, hidden_states, top_k_index, top_k_weights):
     `act_fn(gate) * up` with gate = first half; returns (T, H)."""
     k = top_k_index.shape[-1]
     eid, idx, off = flatten_sort_count(top_k_index, num_experts=self.num_experts)
-    gate_up = parallel_linear(hidden_states, self.gate_up_proj.transpose(1, 2), k, eid, idx, off,
-                              grouped_in=False, grouped_out=True)
-    h = _glu(gate_up, self.act_fn, gate_first=True)
-    return parallel_linear(h, self.down_proj.transpose(1, 2), 1, eid, idx, off,
-                           grouped_in=True, grouped_out=False, gates=top_k_weights.to(h.dtype))
+    return _gated_mlp(hidden_states, self.gate_up_proj, self.down_proj, k, eid, idx, off, top_k_weights, self.act_fn)
 
 
 def patch_experts_class(cls):
@@ -108,11 +121,8 @@ try:
             weights, selected = torch.topk(weights, self.router.top_k, dim=-1)
             weights = (weights / weights.sum(dim=-1, keepdim=True)).to(tokens.dtype)
             eid, idx, off = flatten_sort_count(selected, num_experts=self.router.num_experts)
-            pre = parallel_linear(tokens, self.input_linear.weight.transpose(2, 1), self.router.top_k,
-                                  eid, idx, off, grouped_in=False, grouped_out=True)
-            h = _glu(pre, self.activation, gate_first=True)
-            out = parallel_linear(h, self.output_linear.weight.transpose(2, 1), 1, eid, idx, off,
-                                  grouped_in=True, grouped_out=False, gates=weights)
+            out = _gated_mlp(tokens, self.input_linear.weight, self.output_linear.weight, self.router.top_k,
+                             eid, idx, off, weights, self.activation)
             return out.view(bsz, length, emb_size), router_logits
         top_k_index, top_k_weights, _ = self.router(tokens)
         out = experts_forward(self.experts, tokens, top_k_index, top_k_weights)
