@@ -1,7 +1,8 @@
 // bf16 / fp16 MFMA paths of scatter2scatter and groupXtY for gfx950.
 //
-// One workgroup owns one BM x BN output tile that never straddles two experts and walks the
-// contraction in slices of 64: global -> registers -> LDS (double buffered) -> MFMA 32x32x16.
+// One workgroup owns one BM x BN output tile that never straddles two experts and walks the contraction in
+// slices of 64: global -> LDS directly (double buffered, or a ring of stages for the memory-bound small-row
+// classes) -> MFMA 32x32x16 -> LDS-staged epilogue with 16-byte global accesses.
 // Operands whose contraction axis is contiguous in memory ("direct": gathered X rows, weights stored
 // (N,K)) sit in LDS as [row][64] with a 16-byte XOR swizzle and are read with ds_read_b128; operands
 // whose contraction axis is strided ("transposed": weights stored (K,N), both operands of X^T dY) sit
@@ -11,18 +12,14 @@
 // Counterparts in the reference: _scatter2scatter + _compute_expert_block
 // (scattermoe/kernels/ops.py:11-42, 50-118) and _groupXtY + _xty_and_bias (ops.py:242-366).
 #include "common.hpp"
-#ifndef SMOE_RING_BELOW
-#define SMOE_RING_BELOW 24
-#endif
-#ifndef SMOE_GM
-#define SMOE_GM 4
-#endif
-#ifndef SMOE_GMX
-#define SMOE_GMX 1000000
-#endif
-#ifndef SMOE_OWN
-#define SMOE_OWN 1
-#endif
+
+// Tunables (measured on the Mixtral-shape workload unless noted):
+//   RING_BELOW   average rows per expert under which the 32-row ring-buffered tile classes are used
+//   GM_S2S       row super-tiles per raster band of scatter2scatter (4: +3 % on the layer-2 shaped launches)
+//   GM_XTY       the same for groupXtY (unbanded: bands were neutral there)
+static constexpr int RING_BELOW = 24;
+static constexpr int GM_S2S = 4;
+static constexpr int GM_XTY = 1 << 20;
 #include <type_traits>
 
 namespace smoe {
@@ -811,12 +808,12 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
   __syncthreads();
 
   AOp A;
-  A.rot = SMOE_OWN ? (n_loc * AOp::R / Raster::SN) % AOp::R : 0;      // the row panel has SN sharers
+  A.rot = (n_loc * AOp::R / Raster::SN) % AOp::R;      // the row panel has SN sharers
   const char* Xb = (const char*)a.X;
   const int64_t sxm = a.sxm;
   A.init(Xb, [&](int row) { return (int64_t)sSrc[row] * sxm * 2; });
   BOp B;
-  B.rot = SMOE_OWN ? (m_loc * BOp::R / Raster::SM) % BOp::R : 0;      // the column panel has SM sharers
+  B.rot = (m_loc * BOp::R / Raster::SM) % BOp::R;      // the column panel has SM sharers
   const char* Wb = (const char*)a.W + (int64_t)e * a.swe * 2;
   if (a.glu == 1) {
     // tile column tc -> weight column: wave block tc / WTN, first half of the block from [0, F), second from [F, 2F)
@@ -872,7 +869,7 @@ template <typename T, class TL>
 static int launch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
   const int bn = a.glu == 1 ? TL::BN / 2 : TL::BN;     // output columns per tile
   const int n_tiles = (a.N + bn - 1) / bn;
-  const Raster r = make_raster(max_tiles(a.L, a.E, TL::BM), n_tiles, SMOE_GM);
+  const Raster r = make_raster(max_tiles(a.L, a.E, TL::BM), n_tiles, GM_S2S);
   const int64_t grid = r.grid();
   if (grid > 0x7fffffffLL) { set_error("smoe_scatter2scatter: grid too large"); return SMOE_ERR_RANGE; }
   if constexpr (TL::BN % 128 == 0) {
@@ -890,7 +887,7 @@ static int dispatch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
   const int64_t avg = a.L / a.E;
   if (avg >= 192) return launch_s2s<T, Tile<256, 256, 2, 4>>(a, b_tr, st);
   if (avg >= 96) return launch_s2s<T, Tile<128, 256, 2, 4>>(a, b_tr, st);
-  if (avg >= SMOE_RING_BELOW) return launch_s2s<T, Tile<64, 128, 2, 2, 5>>(a, b_tr, st);
+  if (avg >= RING_BELOW) return launch_s2s<T, Tile<64, 128, 2, 2, 5>>(a, b_tr, st);
   // With one column block per wave the fused forward GLU exists only in its LDS-staged form (16-byte pieces)
   if (a.glu == 1 && !((((uintptr_t)a.Y | (uintptr_t)a.H) & 15) == 0 && ((a.sym | a.shm | a.N) & 7) == 0))
     return SMOE_ERR_UNSUPPORTED;
@@ -1032,7 +1029,7 @@ static int launch_xty(const XtYArgs& a, hipStream_t st) {
   p.db_from_p = k_contig ? 1 : 0;
   const int p_tiles = (p.np + TL::BM - 1) / TL::BM;
   const int q_tiles = (p.nq + TL::BN - 1) / TL::BN;
-  const Raster r = make_raster((int64_t)a.E * p_tiles, q_tiles, SMOE_GMX);
+  const Raster r = make_raster((int64_t)a.E * p_tiles, q_tiles, GM_XTY);
   const int64_t grid = r.grid();
   if (grid > 0x7fffffffLL) { set_error("smoe_groupXtY: grid too large"); return SMOE_ERR_RANGE; }
   hipLaunchKernelGGL((xty_mfma_kernel<T, TL>), dim3((unsigned)grid), dim3(TL::NT), 0, st, p, r, p_tiles);
