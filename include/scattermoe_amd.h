@@ -186,6 +186,17 @@ int smoe_scatter2scatter_glu_bwd(const void* DY, int64_t sdm, int64_t sdk,
                                  const int64_t* eid, const int64_t* idx, const int64_t* off,
                                  int64_t L, int64_t K, int64_t F, int E, int act, int dtype, void* stream);
 
+/*
+ * Router front end: weights, experts = topk(softmax(logits.float(), -1), k) [; weights /= weights.sum(-1)].
+ * Replaces the softmax / topk / renormalise sequence of scattermoe/utils/replace_moe.py:67-71 (the routing of the
+ * Hugging Face blocks the reference patches).  logits (T,E) strides slt,sle, dtype `dtype`; weights_out (T,k)
+ * float32 strides swt,swk, selected in descending order of probability; idx_out (T,k) int64 strides sit,sik.
+ * Among equal probabilities the lowest expert id is selected first.  E <= 512, k <= 64.
+ */
+int smoe_topk_softmax(const void* logits, int64_t slt, int64_t sle, int64_t T, int E, int k, int renormalize,
+                      float* weights_out, int64_t swt, int64_t swk, int64_t* idx_out, int64_t sit, int64_t sik,
+                      int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

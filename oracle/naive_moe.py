@@ -10,6 +10,7 @@ What each function follows in the reference (shawntan/scattermoe):
   naive_token_forward  tests/test_mlp.py:10-26 (dumb_forward) per token, per slot, literal form
   naive_expert_forward the same sum regrouped per expert (gather rows -> 2 linears -> weighted index_add)
   glu / gpt_oss_glu    scattermoe/mlp.py:81-87 ; scattermoe/utils/replace_moe.py:39-43
+  topk_softmax_ref     scattermoe/utils/replace_moe.py:67-71  softmax in float -> topk -> renormalise
 
 How it is pinned (tests/test_oracle.py): the reference stores no golden vectors (its single test
 compares two live computations on unseeded inputs, tests/test_mlp.py:46-49), so every function is
@@ -27,7 +28,7 @@ import torch.nn.functional as F
 __all__ = [
     "route_ref", "scatter2scatter_ref", "group_ref", "group_bwd_W_ref",
     "naive_token_forward", "naive_expert_forward", "glu", "gpt_oss_glu",
-    "module_params", "naive_module_forward",
+    "module_params", "naive_module_forward", "topk_softmax_ref",
 ]
 
 
@@ -41,6 +42,21 @@ def route_ref(expert_idxs, num_experts):
     counts = np.bincount(flat, minlength=num_experts).astype(np.int64)
     return (torch.from_numpy(flat[order].copy()), torch.from_numpy(order),
             torch.from_numpy(np.cumsum(counts)))
+
+
+def topk_softmax_ref(logits, k, renormalize=True):
+    """Router front end: float32 softmax over the experts, the k largest probabilities in descending order
+    (lowest expert id first among equals), optionally divided by their sum.  numpy only.
+    Pinned in tests/test_oracle.py against torch.softmax + torch.topk, hand-worked rows and invariants."""
+    z = np.asarray(torch.as_tensor(logits).detach().cpu().float().numpy(), dtype=np.float32)
+    z = z - z.max(axis=-1, keepdims=True)
+    e = np.exp(z, dtype=np.float32)
+    p = e / e.sum(axis=-1, keepdims=True, dtype=np.float32)
+    order = np.argsort(-p, axis=-1, kind="stable")[:, :k].astype(np.int64)
+    w = np.take_along_axis(p, order, axis=-1)
+    if renormalize:
+        w = w / w.sum(axis=-1, keepdims=True, dtype=np.float32)
+    return torch.from_numpy(w.astype(np.float32)), torch.from_numpy(order)
 
 
 # ---------------------------------------------------------------------------------------------------

@@ -194,4 +194,17 @@ int smoe_glu_bwd(const void* pre, int64_t spm, const void* dh, int64_t sdhm, voi
   return launch_glu_bwd(pre, spm, dh, sdhm, dpre, sdpm, rows, (int)f, act, dtype, (hipStream_t)stream);
 }
 
+int smoe_topk_softmax(const void* logits, int64_t slt, int64_t sle, int64_t T, int E, int k, int renormalize,
+                      float* weights_out, int64_t swt, int64_t swk, int64_t* idx_out, int64_t sit, int64_t sik,
+                      int dtype, void* stream) {
+  g_err[0] = 0;
+  if (!dtype_ok(dtype)) { set_error("smoe_topk_softmax: unknown dtype %d", dtype); return SMOE_ERR_DTYPE; }
+  if (T < 0 || E <= 0 || k <= 0 || k > E) { set_error("smoe_topk_softmax: bad sizes"); return SMOE_ERR_SHAPE; }
+  if (E > 512 || k > 64) { set_error("smoe_topk_softmax: at most 512 experts and top-64"); return SMOE_ERR_RANGE; }
+  if (T == 0) return 0;
+  if (!logits || !weights_out || !idx_out) { set_error("smoe_topk_softmax: NULL pointer"); return SMOE_ERR_NULL; }
+  return launch_topk_softmax(logits, slt, sle, weights_out, swt, swk, idx_out, sit, sik, T, E, k, renormalize, dtype,
+                             (hipStream_t)stream);
+}
+
 }  // extern "C"

@@ -169,6 +169,19 @@ class HipBackend:
         return True
 
 
+    @staticmethod
+    def topk_softmax(logits, weights, experts, renormalize):
+        _C.require_gpu(logits, "topk_softmax")
+        lib = _C.load()
+        with torch.cuda.device(logits.device):
+            rc = lib.smoe_topk_softmax(_C.ptr(logits), logits.stride(0), logits.stride(1), logits.size(0),
+                                       logits.size(1), weights.size(1), int(bool(renormalize)),
+                                       _C.ptr(weights), weights.stride(0), weights.stride(1),
+                                       _C.ptr(experts), experts.stride(0), experts.stride(1),
+                                       _C.float_code(logits.dtype), _C.stream_ptr(logits.device))
+        _C.check(rc, "smoe_topk_softmax")
+
+
 _backend = HipBackend()
 
 
@@ -411,3 +424,43 @@ def scatter2scatter_glu_bwd(DY, W, pre, sorted_expert_idxs, sorted_scattered_idx
     dh = scatter2scatter(DY, W, sorted_expert_idxs, sorted_scattered_idxs, 1, x_grouped=True, y_grouped=True,
                          expert_offsets=expert_offsets)
     return glu_bwd(pre, dh, act)
+
+
+class _TopkSoftmax(torch.autograd.Function):
+    """Forward in one launch; backward is the chain rule of gather -> (renormalise) -> softmax written with
+    torch ops on the (T, E) probabilities, which are recomputed from the logits."""
+
+    @staticmethod
+    def forward(ctx, logits, k, renormalize):
+        T, E = logits.shape
+        weights = torch.empty((T, k), dtype=torch.float32, device=logits.device)
+        experts = torch.empty((T, k), dtype=torch.int64, device=logits.device)
+        _backend.topk_softmax(logits, weights, experts, renormalize)
+        ctx.save_for_backward(logits, weights, experts)
+        ctx.renormalize = renormalize
+        ctx.mark_non_differentiable(experts)
+        return weights, experts
+
+    @staticmethod
+    def backward(ctx, d_weights, _):
+        logits, weights, experts = ctx.saved_tensors
+        p = torch.softmax(logits.float(), dim=-1)
+        d_sel = d_weights.float()
+        if ctx.renormalize:
+            s = p.gather(1, experts).sum(-1, keepdim=True)
+            d_sel = (d_sel - (d_sel * weights).sum(-1, keepdim=True)) / s
+        d_p = torch.zeros_like(p).scatter_(1, experts, d_sel)
+        d_logits = p * (d_p - (d_p * p).sum(-1, keepdim=True))
+        return d_logits.to(logits.dtype), None, None
+
+
+def topk_softmax(router_logits, k, renormalize=True):
+    """`w, i = topk(softmax(router_logits.float(), -1), k)`, then `w /= w.sum(-1, keepdim=True)` when
+    `renormalize` (the routing of scattermoe/utils/replace_moe.py:67-71), in one launch.  Returns float32
+    weights (T, k), in descending order, and int64 expert ids (T, k); equal probabilities are taken lowest
+    expert id first."""
+    if router_logits.dim() != 2:
+        raise ValueError("router_logits must be (tokens, experts)")
+    if not 0 < k <= router_logits.size(1):
+        raise ValueError("k must be in 1..num_experts")
+    return _TopkSoftmax.apply(router_logits, k, renormalize)

@@ -117,9 +117,8 @@ try:
         if hasattr(self, "input_linear"):
             # 4.x layout: router.layer + input_linear / output_linear, returns (output, router_logits)
             router_logits = self.router.layer(tokens)
-            weights = F.softmax(router_logits, dim=1, dtype=torch.float)
-            weights, selected = torch.topk(weights, self.router.top_k, dim=-1)
-            weights = (weights / weights.sum(dim=-1, keepdim=True)).to(tokens.dtype)
+            weights, selected = ops.topk_softmax(router_logits, self.router.top_k, renormalize=True)  # one launch
+            weights = weights.to(tokens.dtype)
             eid, idx, off = flatten_sort_count(selected, num_experts=self.router.num_experts)
             out = _gated_mlp(tokens, self.input_linear.weight, self.output_linear.weight, self.router.top_k,
                              eid, idx, off, weights, self.activation)

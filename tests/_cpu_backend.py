@@ -54,3 +54,8 @@ class OracleBackend:
         s = torch.sigmoid(gate)
         d_lin, d_gate = dh.float() * gate * s, dh.float() * lin * s * (1 + gate * (1 - s))
         dpre.copy_(torch.cat([d_gate, d_lin] if act & 1 else [d_lin, d_gate], dim=-1))
+
+    @staticmethod
+    def topk_softmax(logits, weights, experts, renormalize):
+        w, i = oracle.topk_softmax_ref(logits, weights.size(1), renormalize)
+        weights.copy_(w); experts.copy_(i)

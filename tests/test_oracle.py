@@ -257,3 +257,38 @@ def test_against_huggingface_expert_loops():
         got = oracle.naive_expert_forward(x, p, experts, o.gate_up_proj.transpose(1, 2), o.down_proj.transpose(1, 2),
                                           oracle.gpt_oss_glu(o.alpha, o.limit), o.gate_up_proj_bias, o.down_proj_bias)
     assert torch.allclose(got, want, atol=1e-5)
+
+
+# ---------------------------------------------------------------------------------------------------
+# router front end
+# ---------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("T,E,k", [(1, 8, 2), (33, 8, 2), (64, 32, 4), (17, 128, 8), (5, 300, 3), (4, 4, 4)])
+@pytest.mark.parametrize("renorm", [True, False])
+def test_topk_softmax_matches_library_routines(T, E, k, renorm):
+    logits = torch.randn(T, E, generator=torch.Generator().manual_seed(T * E + k)) * 3
+    w, i = oracle.topk_softmax_ref(logits, k, renorm)
+    p = torch.softmax(logits.float(), dim=-1)
+    tw, ti = torch.topk(p, k, dim=-1)
+    if renorm:
+        tw = tw / tw.sum(-1, keepdim=True)
+    assert torch.equal(i, ti)                       # random floats: no ties, so the order is fixed
+    torch.testing.assert_close(w, tw, rtol=1e-5, atol=1e-7)
+
+
+def test_topk_softmax_hand_worked_and_ties():
+    # logits ln(1), ln(2), ln(3), ln(4): probabilities 0.1 .. 0.4
+    logits = torch.log(torch.tensor([[1.0, 2.0, 3.0, 4.0]]))
+    w, i = oracle.topk_softmax_ref(logits, 2, renormalize=False)
+    assert i.tolist() == [[3, 2]]
+    torch.testing.assert_close(w, torch.tensor([[0.4, 0.3]]), rtol=1e-6, atol=0)
+    w, i = oracle.topk_softmax_ref(logits, 2, renormalize=True)
+    torch.testing.assert_close(w, torch.tensor([[4 / 7, 3 / 7]]), rtol=1e-6, atol=0)
+    # all equal: lowest ids first, uniform weights; shifting the logits changes nothing
+    w, i = oracle.topk_softmax_ref(torch.zeros(2, 6), 3, renormalize=False)
+    assert i.tolist() == [[0, 1, 2]] * 2 and torch.allclose(w, torch.full((2, 3), 1 / 6))
+    a = oracle.topk_softmax_ref(logits + 50.0, 3)
+    b = oracle.topk_softmax_ref(logits, 3)
+    assert torch.equal(a[1], b[1]) and torch.allclose(a[0], b[0], rtol=1e-5)
+    # k = E without renormalisation is the whole softmax, sorted
+    w, i = oracle.topk_softmax_ref(logits, 4, renormalize=False)
+    assert abs(float(w.sum()) - 1.0) < 1e-6 and i.tolist() == [[3, 2, 1, 0]]

@@ -110,6 +110,37 @@ def test_mixtral_style_experts_and_granite_block(cpu_backend):
     assert got_blk.shape == (2, 5, d) and torch.allclose(got_blk, want_blk, atol=1e-5)
 
 
+def test_granite_block_of_transformers_4(cpu_backend):
+    """The layout the reference patched (router.layer + input_linear / output_linear, replace_moe.py:60-95) is gone
+    from transformers 5.x; a stand-in with those attributes checks that path, router front end included."""
+    from types import SimpleNamespace
+    src = __import__("scattermoe_amd.utils.replace_moe", fromlist=["x"])
+    T, E, k, d, f = 12, 4, 2, 16, 24
+    g = torch.Generator().manual_seed(8)
+    layer = torch.nn.Linear(d, E, bias=False)
+    w_in = torch.nn.Parameter(torch.randn(E, 2 * f, d, generator=g) * 0.3)
+    w_out = torch.nn.Parameter(torch.randn(E, d, f, generator=g) * 0.3)
+    blk = SimpleNamespace(router=SimpleNamespace(layer=layer, top_k=k, num_experts=E),
+                          input_linear=SimpleNamespace(weight=w_in), output_linear=SimpleNamespace(weight=w_out),
+                          activation=torch.nn.SiLU())
+    xin = torch.randn(3, 4, d, generator=g, requires_grad=True)
+    got, logits = src.granite_moe_forward(blk, xin)
+    tokens = xin.reshape(-1, d)
+    p = torch.softmax(layer(tokens).float(), -1)
+    w, sel = torch.topk(p, k)
+    w = w / w.sum(-1, keepdim=True)
+    want = torch.zeros(T, d)
+    for e in range(E):
+        pos, tok = torch.where((sel == e).T)
+        gate, up = torch.nn.functional.linear(tokens[tok], w_in[e]).chunk(2, dim=-1)
+        o = torch.nn.functional.linear(torch.nn.functional.silu(gate) * up, w_out[e])
+        want = want.index_add(0, tok, o * w[tok, pos, None])
+    assert logits.shape == (T, E) and torch.allclose(got.reshape(T, d), want, atol=1e-5)
+    params = [xin, layer.weight, w_in, w_out]
+    for a, b in zip(_grads(got, params), _grads(want.view(3, 4, d), params)):
+        assert torch.allclose(a, b, atol=1e-4)
+
+
 def _hf_experts_loop(m, x, index, weights):
     out = torch.zeros_like(x)
     for e in range(m.num_experts):
