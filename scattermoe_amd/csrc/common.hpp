@@ -154,6 +154,7 @@ int launch_xty_generic(const XtYArgs& a, int dtype, hipStream_t st);
 int launch_group(const GroupArgs& a, int dtype, hipStream_t st);
 // MFMA paths return 1 if they took the call, 0 if the shape/layout is not theirs, <0 / >1 never.
 bool try_s2s_mfma(const S2SArgs& a, int dtype, hipStream_t st, int& rc);
+bool try_s2s_rowdot(const S2SArgs& a, int dtype, hipStream_t st, int& rc);   // few-row launches; after try_s2s_mfma's checks
 bool try_xty_mfma(const XtYArgs& a, int dtype, hipStream_t st, int& rc);
 
 int launch_combine(const void* Y, int64_t sy, const void* G, int64_t sgt, int64_t sgk, void* O, int64_t so,

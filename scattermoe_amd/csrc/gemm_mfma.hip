@@ -14,10 +14,14 @@
 #include "common.hpp"
 
 // Tunables (measured on the Mixtral-shape workload unless noted):
-//   RING_BELOW   average rows per expert under which the 32-row ring-buffered tile classes are used
+//   ROWS*_BELOW  average rows per expert under which the 32-, 64-, 128- and 256-row ring-buffered tile classes
+//                are used (weight-streaming regime, Mixtral expert shapes with 64..1536 tokens; from there on
+//                the 256x256 two-stage tile)
+//   GM_RING      tile rows that visit a tile column back to back in the ring classes' order (1: -15 %, 4: -4 %)
 //   GM_S2S       row super-tiles per raster band of scatter2scatter (4: +3 % on the layer-2 shaped launches)
 //   GM_XTY       the same for groupXtY (unbanded: bands were neutral there)
-static constexpr int RING_BELOW = 24;
+static constexpr int ROWS32_BELOW = 24, ROWS64_BELOW = 48, ROWS128_BELOW = 112, ROWS256_BELOW = 224;
+static constexpr int GM_RING = 8;
 static constexpr int GM_S2S = 4;
 static constexpr int GM_XTY = 1 << 20;
 #include <type_traits>
@@ -739,11 +743,20 @@ __device__ __forceinline__ void epilogue_glu_bwd_staged(const f32x16 (&acc)[TL::
 struct Raster {
   static constexpr int SM = 8, SN = 4;
   int m_tiles, n_tiles, m_supers, n_supers, supers, gm;
+  int striped;                             // 1: column-striped order of the memory-bound classes (see make_striped)
   int64_t grid_size;                       // host side only: number of workgroups (may exceed what a launch takes)
   __host__ int64_t grid() const { return grid_size; }
   // (ml, nl): position of the tile inside its super tile
   __device__ __forceinline__ bool map(int pid, int& m, int& n, int& ml, int& nl) const {
     const int x = pid & 7, i = pid >> 3;
+    if (striped) {
+      // XCD x owns the tile columns n = x (mod 8) of every tile row; rows slowest, in groups of gm
+      const int m_lo = i % gm, j = i / gm;
+      m = (j / n_supers) * gm + m_lo;
+      n = (j % n_supers) * 8 + x;
+      ml = nl = 0;
+      return m < m_tiles && n < n_tiles;
+    }
     const int s = (i / (SM * SN)) * 8 + x, r = i % (SM * SN);
     if (s >= supers) return false;
     ml = r % SM;
@@ -767,10 +780,29 @@ static Raster make_raster(int64_t m_tiles, int n_tiles, int gm) {
   r.n_tiles = n_tiles;
   r.m_supers = (int)((m_tiles + Raster::SM - 1) / Raster::SM);
   r.n_supers = (n_tiles + Raster::SN - 1) / Raster::SN;
+  r.striped = 0;
   r.gm = gm < 1 ? 1 : (gm > r.m_supers ? r.m_supers : gm);
   const int64_t supers = (int64_t)r.m_supers * r.n_supers;
   r.grid_size = (supers + 7) / 8 * 8 * Raster::SM * Raster::SN;
   r.supers = supers > 0x7fffffffLL ? 0x7fffffff : (int)supers;   // such a grid is rejected by the launchers
+  return r;
+}
+
+// Order of the memory-bound (ring) classes.  The grid covers an upper bound of the tile rows, so some rows are
+// empty, and which ones is known only on the device: every XCD therefore takes the same share of every tile row
+// (its own residue class of tile columns), and the empty rows, which come last, cost nothing but their launch.
+// `gm` consecutive tile rows visit a tile column back to back on one XCD, so that an expert with several tile
+// rows finds its weight panel in that XCD's L2.
+static Raster make_striped(int64_t m_tiles, int n_tiles, int gm) {
+  Raster r;
+  r.striped = 1;
+  r.m_tiles = (int)m_tiles;
+  r.n_tiles = n_tiles;
+  r.gm = gm < 1 ? 1 : (gm > m_tiles ? (int)m_tiles : gm);
+  r.n_supers = (n_tiles + 7) / 8;                                        // tile columns per XCD
+  r.m_supers = (int)((m_tiles + r.gm - 1) / r.gm);                       // groups of tile rows
+  r.supers = 0;
+  r.grid_size = (int64_t)r.m_supers * r.gm * r.n_supers * 8;
   return r;
 }
 
@@ -869,9 +901,10 @@ template <typename T, class TL>
 static int launch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
   const int bn = a.glu == 1 ? TL::BN / 2 : TL::BN;     // output columns per tile
   const int n_tiles = (a.N + bn - 1) / bn;
-  const Raster r = make_raster(max_tiles(a.L, a.E, TL::BM), n_tiles, GM_S2S);
+  const int64_t m_tiles = max_tiles(a.L, a.E, TL::BM);
+  const Raster r = TL::NS > 2 ? make_striped(m_tiles, n_tiles, GM_RING) : make_raster(m_tiles, n_tiles, GM_S2S);
   const int64_t grid = r.grid();
-  if (grid > 0x7fffffffLL) { set_error("smoe_scatter2scatter: grid too large"); return SMOE_ERR_RANGE; }
+  if (grid > 0x7fffffffLL || m_tiles > 0x7fffffffLL) { set_error("smoe_scatter2scatter: grid too large"); return SMOE_ERR_RANGE; }
   if constexpr (TL::BN % 128 == 0) {
     if (b_tr) {
       hipLaunchKernelGGL((s2s_mfma_kernel<T, TL, true>), dim3((unsigned)grid), dim3(TL::NT), 0, st, a, r);
@@ -885,14 +918,16 @@ static int launch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
 template <typename T>
 static int dispatch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
   const int64_t avg = a.L / a.E;
-  if (avg >= 192) return launch_s2s<T, Tile<256, 256, 2, 4>>(a, b_tr, st);
-  if (avg >= 96) return launch_s2s<T, Tile<128, 256, 2, 4>>(a, b_tr, st);
-  if (avg >= RING_BELOW) return launch_s2s<T, Tile<64, 128, 2, 2, 5>>(a, b_tr, st);
+  if (avg >= ROWS256_BELOW) return launch_s2s<T, Tile<256, 256, 2, 4>>(a, b_tr, st);
+  // Below that the launch is a stream over the weights: ring-buffered classes, tile height by rows per expert
+  if (avg >= ROWS128_BELOW) return launch_s2s<T, Tile<256, 128, 4, 2, 3>>(a, b_tr, st);
+  if (avg >= ROWS32_BELOW && avg < ROWS64_BELOW) return launch_s2s<T, Tile<64, 128, 2, 2, 5>>(a, b_tr, st);
   // With one column block per wave the fused forward GLU exists only in its LDS-staged form (16-byte pieces)
   if (a.glu == 1 && !((((uintptr_t)a.Y | (uintptr_t)a.H) & 15) == 0 && ((a.sym | a.shm | a.N) & 7) == 0))
     return SMOE_ERR_UNSUPPORTED;
-  // Memory-bound class.  With few output columns the 128-wide tiles do not give every CU a workgroup, and what
-  // counts is bytes in flight across the chip: narrower tiles (K-contiguous weights only) restore the count.
+  if (avg >= ROWS64_BELOW) return launch_s2s<T, Tile<128, 128, 2, 4, 3>>(a, b_tr, st);
+  // With few output columns the 128-wide tiles do not give every CU a workgroup, and what counts is bytes in
+  // flight across the chip: narrower tiles (K-contiguous weights only) restore the count.
   const int64_t wgs128 = max_tiles(a.L, a.E, 32) * ((a.N + 127) / 128);
   if (!b_tr && wgs128 < 96) return launch_s2s<T, Tile<32, 32, 1, 1, 8>>(a, b_tr, st);
   if (!b_tr && wgs128 < 192) return launch_s2s<T, Tile<32, 64, 1, 2, 6>>(a, b_tr, st);
@@ -918,6 +953,7 @@ bool try_s2s_mfma(const S2SArgs& a, int dtype, hipStream_t st, int& rc) {
   const int64_t w_cols = a.glu == 1 ? 2 * (int64_t)a.N : a.N;
   if (b_tr ? !fits_u32(BK * a.swk * 2 + w_cols * 2) : !fits_u32((w_cols - 1) * a.swn * 2 + (int64_t)a.K * 2))
     return false;
+  if (!b_tr && try_s2s_rowdot(a, dtype, st, rc)) return true;
   rc = dtype == SMOE_BF16 ? dispatch_s2s<bf16_t>(a, b_tr, st) : dispatch_s2s<f16_t>(a, b_tr, st);
   return true;
 }

@@ -1,0 +1,191 @@
+// scatter2scatter for a handful of rows (single-token and few-token decode): every weight element is used by at
+// most four rows, so the launch is a stream over the weights of the experts that were hit and nothing else
+// matters.  No LDS tiles and no MFMA: each wave reads whole 16-byte pieces of K-contiguous weight rows with
+// plain coalesced loads (a wave instruction covers 1 KB of one weight row), multiplies them with the matching
+// pieces of up to four input rows by packed dot products, and the partial sums are reduced across lanes once at
+// the end.  Many small waves per CU keep far more bytes in flight than the ring-buffered MFMA tiles can.
+//
+// Work split: a workgroup (4 waves) owns C = 8 output columns of one tile of up to R = 4 expert-sorted rows; its
+// waves take the contraction pieces round-robin (piece p of 512 elements goes to wave p % 4), so the four waves
+// together read 4 KB runs of each weight row.  A workgroup walks `gpw` consecutive column groups.
+//
+// Counterparts in the reference: _single2scatter (scattermoe/kernels/single.py:5-59), and _scatter2scatter
+// (scattermoe/kernels/ops.py:50-118) for the row/column conventions, bias and the fused GLU of mlp.py:81-87.
+#include "common.hpp"
+
+namespace smoe {
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T> struct Pair;
+template <> struct Pair<bf16_t> {
+  typedef __bf16 v2 __attribute__((ext_vector_type(2)));
+  static __device__ __forceinline__ float dot(unsigned a, unsigned b, float c) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2, a), __builtin_bit_cast(v2, b), c, false);
+  }
+};
+template <> struct Pair<f16_t> {
+  typedef _Float16 v2 __attribute__((ext_vector_type(2)));
+  static __device__ __forceinline__ float dot(unsigned a, unsigned b, float c) {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(v2, a), __builtin_bit_cast(v2, b), c, false);
+  }
+};
+
+// Sum each of the N = 32 per-lane values over the 64 lanes of the wave with 32 exchanges: every step halves the
+// number of values a lane carries (the lane keeps the half selected by one bit of its id and adds the partner's
+// copy of it).  Afterwards lanes 2j and 2j+1 hold the total of value j in v[0].
+template <int HALF, int OFF, int N>
+__device__ __forceinline__ void transpose_sum_step(float (&v)[N], int lane) {
+  const bool up = (lane & OFF) != 0;
+#pragma unroll
+  for (int i = 0; i < HALF; ++i) {
+    const float keep = up ? v[i + HALF] : v[i];
+    const float send = up ? v[i] : v[i + HALF];
+    v[i] = keep + __shfl_xor(send, OFF, 64);
+  }
+  if constexpr (HALF > 1) transpose_sum_step<HALF / 2, OFF / 2>(v, lane);
+}
+template <int N>
+__device__ __forceinline__ void wave_transpose_sum(float (&v)[N]) {
+  static_assert(N == 32, "written for 32 values over 64 lanes");
+  transpose_sum_step<N / 2, 32>(v, lane_id());
+  v[0] += __shfl_xor(v[0], 1, 64);
+}
+
+static constexpr int ROWDOT_MAX_ROWS = 8;   // launches with more rows than this go to the MFMA tiles
+static constexpr int RD_R = 4;        // rows per tile
+static constexpr int RD_C = 8;        // columns per workgroup pass
+static constexpr int RD_WAVES = 4;
+static constexpr int RD_PIECE = 512;  // contraction elements one wave instruction covers (64 lanes x 8)
+
+template <typename T, bool GLU>
+__global__ __launch_bounds__(RD_WAVES * 64) void s2s_rowdot_kernel(S2SArgs a, int n_groups, int gpw) {
+  constexpr int R = RD_R, C = RD_C;
+  __shared__ float part[RD_WAVES][R * C];
+  const int wave = threadIdx.x >> 6, lane = lane_id();
+  int e, row0, rows;
+  if (!find_tile<R>(a.off, a.E, blockIdx.y, e, row0, rows)) return;
+
+  // source rows of X and destination rows of Y (uniform over the workgroup)
+  int64_t xoff[R], dst[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int64_t n = row0 + (r < rows ? r : rows - 1);
+    int64_t src = n, d = n;
+    if (!a.x_grouped || !a.y_grouped) {
+      const int64_t i = a.idx[n];
+      if (!a.x_grouped) src = i / a.fan_out;
+      if (!a.y_grouped) d = i;
+    }
+    xoff[r] = src * a.sxm * 2;
+    dst[r] = d;
+  }
+  const char* Xb = (const char*)a.X;
+  const char* Wb = (const char*)a.W + (int64_t)e * a.swe * 2;
+  const T* bias = a.b ? (const T*)a.b + (int64_t)e * a.sbe : nullptr;
+  const int F = a.N;                         // GLU: hidden width (the weights have 2F columns)
+  const int K = a.K;
+
+  for (int g = blockIdx.x * gpw; g < min(n_groups, (int)(blockIdx.x + 1) * gpw); ++g) {
+    // column c of the pass -> weight column
+    int col[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      if (GLU) {
+        const int hc = g * (C / 2) + c % (C / 2);
+        col[c] = hc < F ? hc + (c >= C / 2 ? F : 0) : 0;
+      } else {
+        const int n = g * C + c;
+        col[c] = n < F ? n : 0;
+      }
+    }
+    const char* wp[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) wp[c] = Wb + (int64_t)col[c] * a.swn * 2;
+    float acc[R * C];
+#pragma unroll
+    for (int i = 0; i < R * C; ++i) acc[i] = 0.0f;
+
+    for (int k = (wave * 64 + lane) * 8; k < K; k += RD_WAVES * RD_PIECE) {
+      u32x4 w[C], x[R];
+#pragma unroll
+      for (int c = 0; c < C; ++c) w[c] = *(const u32x4*)(wp[c] + (int64_t)k * 2);
+#pragma unroll
+      for (int r = 0; r < R; ++r) x[r] = *(const u32x4*)(Xb + xoff[r] + (int64_t)k * 2);
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) acc[r * C + c] = Pair<T>::dot(x[r][q], w[c][q], acc[r * C + c]);
+    }
+
+    wave_transpose_sum<R * C>(acc);
+    __syncthreads();                               // the previous pass has read `part`
+    if ((lane & 1) == 0) part[wave][lane >> 1] = acc[0];
+    __syncthreads();
+    if (threadIdx.x < R * C) {
+      float v = 0.0f;
+#pragma unroll
+      for (int w_ = 0; w_ < RD_WAVES; ++w_) v += part[w_][threadIdx.x];
+      part[0][threadIdx.x] = v;                    // only this thread read column threadIdx.x of `part`
+    }
+    __syncthreads();
+    if (!GLU) {
+      if (threadIdx.x < R * C) {
+        const int r = threadIdx.x / C, c = threadIdx.x % C;
+        const int n = g * C + c;
+        if (r < rows && n < F) {
+          float v = part[0][threadIdx.x];
+          if (bias != nullptr) v += to_f32(bias[(int64_t)n * a.sbn]);
+          ((T*)a.Y)[dst[r] * a.sym + n] = from_f32<T>(v);
+        }
+      }
+    } else {
+      // both halves are rounded to the storage type first and the hidden value is computed from the rounded values
+      if (threadIdx.x < R * (C / 2)) {
+        const int r = threadIdx.x / (C / 2), c = threadIdx.x % (C / 2);
+        const int n = g * (C / 2) + c;
+        if (r < rows && n < F) {
+          float v1 = part[0][r * C + c], v2 = part[0][r * C + C / 2 + c];
+          if (bias != nullptr) {
+            v1 += to_f32(bias[(int64_t)n * a.sbn]);
+            v2 += to_f32(bias[(int64_t)(F + n) * a.sbn]);
+          }
+          const T first = from_f32<T>(v1), second = from_f32<T>(v2);
+          const bool gf = (a.act & 1) != 0;
+          const float lin = to_f32(gf ? second : first), gat = to_f32(gf ? first : second);
+          const int64_t row = row0 + r;            // the fused form works on rows in grouped order
+          if (a.Y != nullptr) {
+            ((T*)a.Y)[row * a.sym + n] = first;
+            ((T*)a.Y)[row * a.sym + F + n] = second;
+          }
+          ((T*)a.H)[row * a.shm + n] = from_f32<T>(glu_h(a.act, gat, lin));
+        }
+      }
+    }
+  }
+}
+
+// Called with the operand checks of the MFMA path already done (K-contiguous weights, 16-byte aligned rows,
+// K a multiple of 8).  Returns false when the shape is not this kernel's.
+bool try_s2s_rowdot(const S2SArgs& a, int dtype, hipStream_t st, int& rc) {
+  if (a.glu == 2 || a.L > ROWDOT_MAX_ROWS) return false;
+  const int64_t m_tiles = max_tiles(a.L, a.E, RD_R);
+  const int n_groups = a.glu == 1 ? (a.N + RD_C / 2 - 1) / (RD_C / 2) : (a.N + RD_C - 1) / RD_C;
+  // enough workgroups to give every CU several, few enough that the tile lookup is amortised
+  int gpw = 1;
+  while (gpw < 8 && m_tiles * ((n_groups + 2 * gpw - 1) / (2 * gpw)) >= 2048) gpw *= 2;
+  const dim3 grid((unsigned)((n_groups + gpw - 1) / gpw), (unsigned)m_tiles), block(RD_WAVES * 64);
+  if (dtype == SMOE_BF16) {
+    if (a.glu) hipLaunchKernelGGL((s2s_rowdot_kernel<bf16_t, true>), grid, block, 0, st, a, n_groups, gpw);
+    else hipLaunchKernelGGL((s2s_rowdot_kernel<bf16_t, false>), grid, block, 0, st, a, n_groups, gpw);
+  } else {
+    if (a.glu) hipLaunchKernelGGL((s2s_rowdot_kernel<f16_t, true>), grid, block, 0, st, a, n_groups, gpw);
+    else hipLaunchKernelGGL((s2s_rowdot_kernel<f16_t, false>), grid, block, 0, st, a, n_groups, gpw);
+  }
+  rc = launch_status("s2s_rowdot_kernel");
+  return true;
+}
+
+}  // namespace smoe

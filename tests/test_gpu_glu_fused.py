@@ -18,8 +18,9 @@ DEV = "cuda:0"
 SHAPES = [
     (2048, 4, 2, 256, 384),      # 1024 rows/expert: 256-row tiles, exact multiples
     (1100, 8, 2, 200, 264),      # 275 rows/expert: ragged rows, d % 64 != 0, F % 128 != 0
-    (520, 8, 2, 320, 1000),      # 130 rows/expert: 128-row tiles
-    (130, 8, 3, 448, 72),        # ~49 rows/expert: 64-row ring tiles, F < one tile
+    (520, 8, 2, 320, 1000),      # 130 rows/expert: ring-buffered 256x128 tiles
+    (130, 8, 3, 448, 72),        # ~49 rows/expert: ring-buffered 128x128 tiles, F < one tile
+    (130, 8, 2, 320, 200),       # ~32 rows/expert: 64-row ring tiles
     (40, 8, 2, 192, 136),        # 10 rows/expert: no fused forward kernel (falls back), fused backward
 ]
 
@@ -78,7 +79,7 @@ def test_fused_backward_equals_two_launches(T, E, k, d, F, act, layout, dtype):
 
 
 @pytest.mark.parametrize("bias", [False, True])
-@pytest.mark.parametrize("T,E,k,d,F", SHAPES[:4])
+@pytest.mark.parametrize("T,E,k,d,F", SHAPES[:5])
 def test_module_matches_unfused_chain(T, E, k, d, F, bias):
     """GLUMLP (one autograd node, fused launches) against the chain of ParallelLinear nodes it replaces."""
     torch.manual_seed(1)
