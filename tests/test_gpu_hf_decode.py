@@ -105,3 +105,43 @@ def test_single2scatter_gpu():
         want = torch.stack([x[j if rows == k else 0].float() @ W[e].float() for j, e in enumerate(experts[0])])
         got = single2scatter(x.to(DEV), W.to(DEV), experts.to(DEV))
         _close(got, want, 2e-2, 1e-2)
+
+
+@pytest.mark.parametrize("T", [1, 4, 40])
+def test_decode_forward_replays_from_a_hip_graph(T):
+    """The library allocates, clears and synchronises nothing, so a whole module forward captures into a HIP graph.
+    Every replay (new inputs written into the static buffers, eager work and synchronisations in between) must
+    reproduce the eager result bit for bit.  T = 1 and 4 run the row-dot kernels, T = 40 the ring tiles."""
+    from scattermoe_amd.mlp import GLUMLP
+    from scattermoe_amd.kernels.ops import topk_softmax
+    E, k, d, f = 8, 2, 256, 384
+    torch.manual_seed(7)
+    with torch.device(DEV):
+        m = GLUMLP(d, f, E, k).to(torch.bfloat16)
+    g = torch.Generator().manual_seed(T)
+    x = torch.randn(T, d, generator=g).to(torch.bfloat16).to(DEV)
+    logits = torch.randn(T, E, generator=g).to(DEV)
+
+    def step(xx, ll):
+        w, i = topk_softmax(ll, k)
+        return m(xx, w.to(torch.bfloat16), i)
+
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                step(x, logits)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            y_static = step(x, logits)
+        for r in range(4):
+            x.copy_(torch.randn(T, d, generator=g).to(torch.bfloat16))
+            logits.copy_(torch.randn(T, E, generator=g))
+            graph.replay()
+            torch.cuda.synchronize()
+            got = y_static.clone()
+            want = step(x, logits)                       # eager work between the replays
+            torch.cuda.synchronize()
+            assert torch.equal(got, want), "replay %d differs from the eager result" % r
