@@ -36,6 +36,9 @@ def parse():
     ap.add_argument("--workload", default="c2")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-tokens", type=int, default=0, help="token count of the CPU sample (default T/16)")
+    ap.add_argument("--decode", type=int, default=0, metavar="T",
+                    help="forward-only latency of one layer at T tokens (decode regime of the workload's expert "
+                         "shape); prints its own JSON line with an HBM roofline")
     ap.add_argument("--profile-kernel", default="",
                     help="run ONLY one kernel of the workload `steps` times (for rocprofv3 --pmc): "
                          "l1fwd | l2fwd | l1dx | l2dx | l1dw | l2dw | copy (a 256 MiB device copy of known size)")
@@ -155,6 +158,42 @@ def profile_one_kernel(args, cfg, torch, ops):
     torch.cuda.synchronize()
 
 
+def decode_line(args, cfg, torch):
+    """One MoE layer forward at `--decode T` tokens under no_grad: a stream over the weights of the experts hit."""
+    from torch import nn
+    from scattermoe_amd.mlp import GLUMLP, MLP
+    dev, dt, T = torch.device("cuda:0"), cfg.dtype, args.decode
+    g = torch.Generator(device=dev).manual_seed(T)
+    p, experts = torch.topk(torch.softmax(torch.randn(T, cfg.E, generator=g, device=dev), -1), cfg.k)
+    p = (p / p.sum(-1, keepdim=True)).to(dt)
+    x = torch.randn(T, cfg.d, generator=g, device=dev).to(dt)
+    cls = GLUMLP if cfg.glu else MLP
+    with torch.device(dev):
+        m = cls(cfg.d, cfg.f, cfg.E, cfg.k, bias=cfg.bias, activation=nn.SiLU() if cfg.glu else nn.GELU()).to(dt)
+    hit = int(experts.unique().numel())
+    with torch.no_grad():
+        for _ in range(args.warmup):
+            m(x, p, experts)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            m(x, p, experts)
+        torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    w_bytes = hit * (3 if cfg.glu else 2) * cfg.d * cfg.f * x.element_size()
+    gbs = w_bytes / (ms * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "moe_mlp_decode_layer_ms", "value": round(ms, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": False, "vs_baseline": None,
+        "dtype": {torch.bfloat16: "bf16", torch.float32: "f32", torch.float16: "f16"}[dt], "data": "synthetic",
+        "config": {"workload": "%s expert shape, forward only, T=%d tokens (d_model=%d d_ff=%d E=%d top_k=%d)" % (
+            cfg.name, T, cfg.d, cfg.f, cfg.E, cfg.k), "tokens": T, "experts_hit": hit},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": 8000.0, "unit": "GB/s",
+                     "frac": round(gbs / 8000.0, 4), "traffic": None,
+                     "bytes": "weights of the experts hit: %d x %d matrices of d_model x d_ff" % (
+                         hit, 3 if cfg.glu else 2)}}))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -178,6 +217,9 @@ def main():
     dtype = cfg.dtype
     if args.profile_kernel:
         profile_one_kernel(args, cfg, torch, ops)
+        return
+    if args.decode:
+        decode_line(args, cfg, torch)
         return
 
     # synthetic inputs, generated on the device with a fixed seed; resident before timing starts
