@@ -100,8 +100,33 @@ def require_gpu(t, what):
             % (what, t.device))
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_ptr(device):
+    """hipStream_t of torch's current stream on `device`, as an integer."""
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index)
     return torch.cuda.current_stream(device).cuda_stream
+
+
+class _NoSwitch:
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def on_device(device):
+    """Context that makes `device` the current HIP device for a launch; free when it already is (the usual case:
+    switching costs several microseconds of host time per launch, which a decode step cannot hide)."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NO_SWITCH
+    return torch.cuda.device(device)
 
 
 def ptr(t):

@@ -31,7 +31,7 @@ class HipBackend:
         L = flat_ids.numel()
         need = lib.smoe_route_workspace_bytes(L, num_experts)
         ws = torch.empty(need, dtype=torch.uint8, device=flat_ids.device) if need else None
-        with torch.cuda.device(flat_ids.device):
+        with _C.on_device(flat_ids.device):
             rc = lib.smoe_route(_C.ptr(flat_ids), _C.index_code(flat_ids.dtype), L, num_experts,
                                 _C.ptr(eid), _C.ptr(idx), _C.ptr(off), _C.ptr(ws), need,
                                 _C.stream_ptr(flat_ids.device))
@@ -41,7 +41,7 @@ class HipBackend:
     def offsets(eid, num_experts, off):
         _C.require_gpu(eid, "expert offsets")
         lib = _C.load()
-        with torch.cuda.device(eid.device):
+        with _C.on_device(eid.device):
             rc = lib.smoe_offsets_from_sorted(_C.ptr(eid), eid.numel(), num_experts, _C.ptr(off),
                                               _C.stream_ptr(eid.device))
         _C.check(rc, "smoe_offsets_from_sorted")
@@ -51,7 +51,7 @@ class HipBackend:
         _C.require_gpu(X, "scatter2scatter")
         lib = _C.load()
         sbe, sbn = (b.stride(0), b.stride(1)) if b is not None else (0, 0)
-        with torch.cuda.device(X.device):
+        with _C.on_device(X.device):
             rc = lib.smoe_scatter2scatter(
                 _C.ptr(X), X.stride(0), X.stride(1),
                 _C.ptr(W), W.stride(0), W.stride(1), W.stride(2),
@@ -67,7 +67,7 @@ class HipBackend:
     def group(A, coeff, Y, idx, fan_out):
         _C.require_gpu(A, "group")
         lib = _C.load()
-        with torch.cuda.device(A.device):
+        with _C.on_device(A.device):
             rc = lib.smoe_group(_C.ptr(A), A.stride(0), A.stride(1), _C.ptr(coeff),
                                 _C.ptr(Y), Y.stride(0), Y.stride(1), _C.ptr(idx),
                                 idx.numel(), A.size(1), fan_out, _C.float_code(A.dtype),
@@ -79,7 +79,7 @@ class HipBackend:
         _C.require_gpu(DY, "group_bwd_W")
         lib = _C.load()
         sdbe, sdbn = (Db.stride(0), Db.stride(1)) if Db is not None else (0, 0)
-        with torch.cuda.device(DY.device):
+        with _C.on_device(DY.device):
             rc = lib.smoe_groupXtY(
                 _C.ptr(DY), DY.stride(0), DY.stride(1),
                 _C.ptr(X), X.stride(0), X.stride(1),
@@ -94,7 +94,7 @@ class HipBackend:
     def combine(Y, gates, out, k):
         _C.require_gpu(Y, "combine")
         lib = _C.load()
-        with torch.cuda.device(Y.device):
+        with _C.on_device(Y.device):
             rc = lib.smoe_combine(_C.ptr(Y), Y.stride(0), _C.ptr(gates), gates.stride(0), gates.stride(1),
                                   _C.ptr(out), out.stride(0), out.size(0), k, Y.size(1),
                                   _C.float_code(Y.dtype), _C.stream_ptr(Y.device))
@@ -104,7 +104,7 @@ class HipBackend:
     def gate_grad(Y, d_out, d_gates, k):
         _C.require_gpu(Y, "gate_grad")
         lib = _C.load()
-        with torch.cuda.device(Y.device):
+        with _C.on_device(Y.device):
             rc = lib.smoe_gate_grad(_C.ptr(Y), Y.stride(0), _C.ptr(d_out), d_out.stride(0),
                                     _C.ptr(d_gates), d_gates.stride(0), d_gates.stride(1),
                                     d_out.size(0), k, Y.size(1), _C.float_code(Y.dtype),
@@ -115,7 +115,7 @@ class HipBackend:
     def glu_fwd(pre, h, act):
         _C.require_gpu(pre, "glu_fwd")
         lib = _C.load()
-        with torch.cuda.device(pre.device):
+        with _C.on_device(pre.device):
             rc = lib.smoe_glu_fwd(_C.ptr(pre), pre.stride(0), _C.ptr(h), h.stride(0), pre.size(0), h.size(1),
                                   act, _C.float_code(pre.dtype), _C.stream_ptr(pre.device))
         _C.check(rc, "smoe_glu_fwd")
@@ -124,7 +124,7 @@ class HipBackend:
     def glu_bwd(pre, dh, dpre, act):
         _C.require_gpu(pre, "glu_bwd")
         lib = _C.load()
-        with torch.cuda.device(pre.device):
+        with _C.on_device(pre.device):
             rc = lib.smoe_glu_bwd(_C.ptr(pre), pre.stride(0), _C.ptr(dh), dh.stride(0), _C.ptr(dpre),
                                   dpre.stride(0), pre.size(0), dh.size(1), act, _C.float_code(pre.dtype),
                                   _C.stream_ptr(pre.device))
@@ -136,7 +136,7 @@ class HipBackend:
         _C.require_gpu(X, "scatter2scatter_glu")
         lib = _C.load()
         sbe, sbn = (b.stride(0), b.stride(1)) if b is not None else (0, 0)
-        with torch.cuda.device(X.device):
+        with _C.on_device(X.device):
             rc = lib.smoe_scatter2scatter_glu(
                 _C.ptr(X), X.stride(0), X.stride(1),
                 _C.ptr(W), W.stride(0), W.stride(1), W.stride(2),
@@ -155,7 +155,7 @@ class HipBackend:
         """Fused layer-2 input gradient + GLU gradient; False when there is no fused kernel for this call."""
         _C.require_gpu(DY, "scatter2scatter_glu_bwd")
         lib = _C.load()
-        with torch.cuda.device(DY.device):
+        with _C.on_device(DY.device):
             rc = lib.smoe_scatter2scatter_glu_bwd(
                 _C.ptr(DY), DY.stride(0), DY.stride(1),
                 _C.ptr(W), W.stride(0), W.stride(1), W.stride(2),
@@ -173,7 +173,7 @@ class HipBackend:
     def topk_softmax(logits, weights, experts, renormalize):
         _C.require_gpu(logits, "topk_softmax")
         lib = _C.load()
-        with torch.cuda.device(logits.device):
+        with _C.on_device(logits.device):
             rc = lib.smoe_topk_softmax(_C.ptr(logits), logits.stride(0), logits.stride(1), logits.size(0),
                                        logits.size(1), weights.size(1), int(bool(renormalize)),
                                        _C.ptr(weights), weights.stride(0), weights.stride(1),

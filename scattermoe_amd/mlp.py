@@ -34,13 +34,12 @@ class _GatedMLP(torch.autograd.Function):
         # w1 (E, 2F, d), w2 (E, d, F): the ParallelExperts parameters; the kernels take the (E, in, out) views
         T = x.size(0)
         need_grad = any(ctx.needs_input_grad[:6])
-        with torch.device(x.device):
-            pre, h = ops.scatter2scatter_glu(x, w1.permute(0, 2, 1), eid, idx, k, b=b1, act=act,
-                                             expert_offsets=off, need_pre=need_grad)
-            expanded = ops.scatter2scatter(h, w2.permute(0, 2, 1), eid, idx, 1, b=b2, x_grouped=True,
-                                           y_grouped=False, expert_offsets=off)
-            kept = expanded.view(T, k, expanded.size(-1))
-            out = ops.combine(kept, gates)
+        pre, h = ops.scatter2scatter_glu(x, w1.permute(0, 2, 1), eid, idx, k, b=b1, act=act,
+                                         expert_offsets=off, need_pre=need_grad)
+        expanded = ops.scatter2scatter(h, w2.permute(0, 2, 1), eid, idx, 1, b=b2, x_grouped=True,
+                                       y_grouped=False, expert_offsets=off)
+        kept = expanded.view(T, k, expanded.size(-1))
+        out = ops.combine(kept, gates)
         if need_grad:
             ctx.save_for_backward(x, w1, b1, w2, b2, gates, eid, idx, off, pre, h, kept)
         ctx.k, ctx.act = k, act
@@ -56,26 +55,25 @@ class _GatedMLP(torch.autograd.Function):
         E = w1.size(0)
         if not grad_out.is_contiguous():
             grad_out = grad_out.contiguous()
-        with torch.device(grad_out.device):
-            d_gates = ops.gate_grad(kept, grad_out) if need_g else None
-            # dY of layer 2 in expert-sorted order, scaled by each row's gate; reuses the expert-output buffer
-            dy = ops.group(grad_out, idx, coeff=gates.reshape(-1).to(grad_out.dtype), fan_out=k,
-                           out=kept.view(-1, kept.size(-1)))
-            d_w2 = d_b2 = None
-            if need_w2 or need_b2:
-                d_w2, d_b2 = ops.group_bwd_W(DY=dy, X=h, expert_offsets=off, E=E, has_bias=b2 is not None)
-                d_w2 = d_w2.permute(0, 2, 1) if need_w2 else None     # back to the parameter layout (E, d, F)
-            d_x = d_w1 = d_b1 = None
-            if need_x or need_w1 or need_b1:
-                dpre = ops.scatter2scatter_glu_bwd(dy, w2, pre, eid, idx, act=act, expert_offsets=off)
-                xg = ops.group(x, idx, fan_out=k)
-                if need_w1 or need_b1:
-                    d_w1, d_b1 = ops.group_bwd_W(DY=dpre, X=xg, expert_offsets=off, E=E, has_bias=b1 is not None)
-                    d_w1 = d_w1.permute(0, 2, 1) if need_w1 else None
-                if need_x:
-                    d_exp = ops.scatter2scatter(dpre, w1, eid, idx, 1, x_grouped=True, y_grouped=False,
-                                                out=xg, expert_offsets=off)
-                    d_x = d_exp if k == 1 else d_exp.view(x.size(0), k, d_exp.size(-1)).sum(-2)
+        d_gates = ops.gate_grad(kept, grad_out) if need_g else None
+        # dY of layer 2 in expert-sorted order, scaled by each row's gate; reuses the expert-output buffer
+        dy = ops.group(grad_out, idx, coeff=gates.reshape(-1).to(grad_out.dtype), fan_out=k,
+                       out=kept.view(-1, kept.size(-1)))
+        d_w2 = d_b2 = None
+        if need_w2 or need_b2:
+            d_w2, d_b2 = ops.group_bwd_W(DY=dy, X=h, expert_offsets=off, E=E, has_bias=b2 is not None)
+            d_w2 = d_w2.permute(0, 2, 1) if need_w2 else None     # back to the parameter layout (E, d, F)
+        d_x = d_w1 = d_b1 = None
+        if need_x or need_w1 or need_b1:
+            dpre = ops.scatter2scatter_glu_bwd(dy, w2, pre, eid, idx, act=act, expert_offsets=off)
+            xg = ops.group(x, idx, fan_out=k)
+            if need_w1 or need_b1:
+                d_w1, d_b1 = ops.group_bwd_W(DY=dpre, X=xg, expert_offsets=off, E=E, has_bias=b1 is not None)
+                d_w1 = d_w1.permute(0, 2, 1) if need_w1 else None
+            if need_x:
+                d_exp = ops.scatter2scatter(dpre, w1, eid, idx, 1, x_grouped=True, y_grouped=False,
+                                            out=xg, expert_offsets=off)
+                d_x = d_exp if k == 1 else d_exp.view(x.size(0), k, d_exp.size(-1)).sum(-2)
         return d_x, d_w1, (d_b1 if need_b1 else None), d_w2, (d_b2 if need_b2 else None), d_gates, \
             None, None, None, None, None
 

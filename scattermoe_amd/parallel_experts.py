@@ -52,16 +52,15 @@ class ParallelLinear(torch.autograd.Function):
                 expert_biases: Optional[torch.Tensor] = None,
                 gates: Optional[torch.Tensor] = None,
                 grouped_in: bool = False, grouped_out: bool = False):
-        with torch.device(x.device):
-            expanded = ops.scatter2scatter(
-                X=x, W=expert_weights, b=expert_biases, k=k,
-                sorted_expert_idxs=sorted_expert_idxs, sorted_scattered_idxs=sorted_scattered_idxs,
-                x_grouped=grouped_in, y_grouped=grouped_out, expert_offsets=expert_offsets)
-            if gates is None:
-                result, kept = expanded, None
-            else:
-                kept = expanded.view(gates.size(0), gates.size(1), expanded.size(-1))
-                result = ops.combine(kept, gates)
+        expanded = ops.scatter2scatter(
+            X=x, W=expert_weights, b=expert_biases, k=k,
+            sorted_expert_idxs=sorted_expert_idxs, sorted_scattered_idxs=sorted_scattered_idxs,
+            x_grouped=grouped_in, y_grouped=grouped_out, expert_offsets=expert_offsets)
+        if gates is None:
+            result, kept = expanded, None
+        else:
+            kept = expanded.view(gates.size(0), gates.size(1), expanded.size(-1))
+            result = ops.combine(kept, gates)
         ctx.save_for_backward(x, expert_weights, expert_biases, sorted_expert_idxs,
                               sorted_scattered_idxs, expert_offsets, gates, kept)
         ctx.k, ctx.grouped_in, ctx.grouped_out = k, grouped_in, grouped_out
@@ -78,40 +77,39 @@ class ParallelLinear(torch.autograd.Function):
         if not grad_out.is_contiguous():
             grad_out = grad_out.contiguous()
 
-        with torch.device(grad_out.device):
-            d_gates = None
-            coeff, coeff_fan, dy_buf = None, 1, None
-            if gates is not None:
-                if need_g:
-                    # (T, k): row dots of every expert output with dY
-                    d_gates = ops.gate_grad(kept, grad_out)
-                coeff, coeff_fan = gates.reshape(-1), gates.size(1)
-                dy_buf = kept.view(-1, kept.size(-1))   # its contents are dead once d_gates exists
+        d_gates = None
+        coeff, coeff_fan, dy_buf = None, 1, None
+        if gates is not None:
+            if need_g:
+                # (T, k): row dots of every expert output with dY
+                d_gates = ops.gate_grad(kept, grad_out)
+            coeff, coeff_fan = gates.reshape(-1), gates.size(1)
+            dy_buf = kept.view(-1, kept.size(-1))   # its contents are dead once d_gates exists
 
-            # dY in expert-sorted order, scaled by the gate of each (token, slot)
-            if grouped_out:
-                dy = grad_out
-            else:
-                dy = ops.group(grad_out, idx, coeff=coeff, fan_out=coeff_fan, out=dy_buf)
+        # dY in expert-sorted order, scaled by the gate of each (token, slot)
+        if grouped_out:
+            dy = grad_out
+        else:
+            dy = ops.group(grad_out, idx, coeff=coeff, fan_out=coeff_fan, out=dy_buf)
 
-            d_w = d_b = None
-            xg = None
-            if need_w or need_b or (need_x and not grouped_in):
-                xg = x if grouped_in else ops.group(x, idx, fan_out=k)
-            if need_w or need_b:
-                d_w, d_b = ops.group_bwd_W(DY=dy, X=xg, expert_offsets=off, E=E, has_bias=bias is not None)
-                if not need_w:
-                    d_w = None
+        d_w = d_b = None
+        xg = None
+        if need_w or need_b or (need_x and not grouped_in):
+            xg = x if grouped_in else ops.group(x, idx, fan_out=k)
+        if need_w or need_b:
+            d_w, d_b = ops.group_bwd_W(DY=dy, X=xg, expert_offsets=off, E=E, has_bias=bias is not None)
+            if not need_w:
+                d_w = None
 
-            d_x = None
-            if need_x:
-                # dX rows: dY @ W[e]^T, written grouped (grouped_in) or scattered back to slot order;
-                # the gathered copy of x is dead by now and is reused as the output buffer
-                d_exp = ops.scatter2scatter(
-                    X=dy, W=W.permute(0, 2, 1), k=1, x_grouped=True, y_grouped=grouped_in,
-                    sorted_expert_idxs=eid, sorted_scattered_idxs=idx,
-                    out=None if grouped_in else xg, expert_offsets=off)
-                d_x = d_exp if k == 1 else d_exp.view(x.size(0), k, d_exp.size(-1)).sum(-2)
+        d_x = None
+        if need_x:
+            # dX rows: dY @ W[e]^T, written grouped (grouped_in) or scattered back to slot order;
+            # the gathered copy of x is dead by now and is reused as the output buffer
+            d_exp = ops.scatter2scatter(
+                X=dy, W=W.permute(0, 2, 1), k=1, x_grouped=True, y_grouped=grouped_in,
+                sorted_expert_idxs=eid, sorted_scattered_idxs=idx,
+                out=None if grouped_in else xg, expert_offsets=off)
+            d_x = d_exp if k == 1 else d_exp.view(x.size(0), k, d_exp.size(-1)).sum(-2)
 
         return d_x, d_w, None, None, None, None, d_b, d_gates, None, None
 
