@@ -95,3 +95,20 @@ def test_leading_dims_and_determinism():
     p, e = torch.topk(torch.softmax(torch.randn(51, 8, device=DEV), -1), 2)
     y1, y2 = m(x, p, e), m(x, p, e)
     assert y1.shape == (3, 17, 64) and torch.equal(y1, y2)
+
+
+@pytest.mark.parametrize("cls,dtype", [(GLUMLP, torch.bfloat16), (GLUMLP, torch.float32), (MLP, torch.float32)])
+def test_empty_batch(cls, dtype):
+    """No tokens: empty output, empty input gradients, zero weight gradients (every expert is empty)."""
+    kw = {} if cls is GLUMLP else {"activation": nn.GELU()}
+    with torch.device(DEV):
+        m = cls(64, 96, 8, 2, **kw).to(dtype)
+    x = torch.empty(0, 64, device=DEV, dtype=dtype, requires_grad=True)
+    p = torch.empty(0, 2, device=DEV, dtype=dtype, requires_grad=True)
+    experts = torch.empty(0, 2, device=DEV, dtype=torch.int64)
+    y = m(x, p, experts)
+    assert y.shape == (0, 64)
+    y.sum().backward()
+    assert x.grad.shape == (0, 64) and p.grad.shape == (0, 2)
+    for prm in m.parameters():
+        assert prm.grad is not None and not prm.grad.isnan().any() and float(prm.grad.abs().max()) == 0.0
