@@ -185,6 +185,78 @@ class HipBackend:
 _backend = HipBackend()
 
 
+# ------------------------------------------------------------------------------------------------
+# Under torch.compile every launch has to be an operator the tracer knows (it cannot look inside a ctypes call).
+# The three kernels of the reference are registered further down under the reference's own operator names; the
+# remaining launches of this build are registered here.  All of them write into buffers the caller allocated.
+# ------------------------------------------------------------------------------------------------
+@torch.library.custom_op("scattermoe::route", mutates_args={"eid", "idx", "off"})
+def _route_op(flat_ids: torch.Tensor, num_experts: int, eid: torch.Tensor, idx: torch.Tensor,
+              off: torch.Tensor) -> None:
+    _backend.route(flat_ids, num_experts, eid, idx, off)
+
+
+@torch.library.custom_op("scattermoe::offsets", mutates_args={"off"})
+def _offsets_op(eid: torch.Tensor, num_experts: int, off: torch.Tensor) -> None:
+    _backend.offsets(eid, num_experts, off)
+
+
+@torch.library.custom_op("scattermoe::combine", mutates_args={"out"})
+def _combine_op(Y: torch.Tensor, gates: torch.Tensor, out: torch.Tensor, k: int) -> None:
+    _backend.combine(Y, gates, out, k)
+
+
+@torch.library.custom_op("scattermoe::gate_grad", mutates_args={"d_gates"})
+def _gate_grad_op(Y: torch.Tensor, d_out: torch.Tensor, d_gates: torch.Tensor, k: int) -> None:
+    _backend.gate_grad(Y, d_out, d_gates, k)
+
+
+@torch.library.custom_op("scattermoe::glu_fwd", mutates_args={"h"})
+def _glu_fwd_op(pre: torch.Tensor, h: torch.Tensor, act: int) -> None:
+    _backend.glu_fwd(pre, h, act)
+
+
+@torch.library.custom_op("scattermoe::glu_bwd", mutates_args={"dpre"})
+def _glu_bwd_op(pre: torch.Tensor, dh: torch.Tensor, dpre: torch.Tensor, act: int) -> None:
+    _backend.glu_bwd(pre, dh, dpre, act)
+
+
+@torch.library.custom_op("scattermoe::topk_softmax", mutates_args={"weights", "experts"})
+def _topk_softmax_op(logits: torch.Tensor, weights: torch.Tensor, experts: torch.Tensor,
+                     renormalize: bool) -> None:
+    _backend.topk_softmax(logits, weights, experts, renormalize)
+
+
+@torch.library.custom_op("scattermoe::scatter2scatter_glu", mutates_args={"pre", "h"})
+def _s2s_glu_op(X: torch.Tensor, W: torch.Tensor, b: Optional[torch.Tensor], pre: Optional[torch.Tensor],
+                h: torch.Tensor, eid: torch.Tensor, idx: torch.Tensor, off: torch.Tensor, k: int,
+                x_grouped: bool, act: int) -> None:
+    if not _backend.s2s_glu(X, W, b, pre, h, eid, idx, off, k, x_grouped, act):   # no fused kernel: two launches
+        tmp = pre if pre is not None else torch.empty((h.size(0), 2 * h.size(1)), dtype=h.dtype, device=h.device)
+        _backend.s2s(X, W, b, tmp, eid, idx, off, k, x_grouped, True)
+        _backend.glu_fwd(tmp, h, act)
+
+
+@torch.library.custom_op("scattermoe::scatter2scatter_glu_bwd", mutates_args={"dpre"})
+def _s2s_glu_bwd_op(DY: torch.Tensor, W: torch.Tensor, pre: torch.Tensor, dpre: torch.Tensor, eid: torch.Tensor,
+                    idx: torch.Tensor, off: torch.Tensor, act: int) -> None:
+    if not _backend.s2s_glu_bwd(DY, W, pre, dpre, eid, idx, off, act):
+        dh = torch.empty((DY.size(0), W.size(2)), dtype=DY.dtype, device=DY.device)
+        _backend.s2s(DY, W, None, dh, eid, idx, off, 1, True, True)
+        _backend.glu_bwd(pre, dh, dpre, act)
+
+
+_COMPILED_OPS = {"route": _route_op, "offsets": _offsets_op, "combine": _combine_op, "gate_grad": _gate_grad_op,
+                 "glu_fwd": _glu_fwd_op, "glu_bwd": _glu_bwd_op, "topk_softmax": _topk_softmax_op}
+
+
+def _launch(name, *args):
+    """`_backend.<name>(*args)`, through the registered operator while a compiler is tracing."""
+    if torch.compiler.is_compiling():
+        return _COMPILED_OPS[name](*args)
+    return getattr(_backend, name)(*args)
+
+
 def _same_dtype(what, ref, *others):
     for t in others:
         if t is not None and t.dtype != ref.dtype:
@@ -209,13 +281,13 @@ def route(expert_idxs: torch.Tensor, num_experts: int):
     eid = torch.empty(L, dtype=torch.int64, device=flat.device)
     idx = torch.empty(L, dtype=torch.int64, device=flat.device)
     off = torch.empty(num_experts, dtype=torch.int64, device=flat.device)
-    _backend.route(flat, num_experts, eid, idx, off)
+    _launch("route", flat, num_experts, eid, idx, off)
     return eid, idx, off
 
 
 def offsets_from_sorted(sorted_expert_idxs: torch.Tensor, num_experts: int):
     off = torch.empty(num_experts, dtype=torch.int64, device=sorted_expert_idxs.device)
-    _backend.offsets(_as_i64(sorted_expert_idxs).contiguous(), num_experts, off)
+    _launch("offsets", _as_i64(sorted_expert_idxs).contiguous(), num_experts, off)
     return off
 
 
@@ -351,7 +423,7 @@ def combine(expanded, gates):
     assert gates.shape == (T, k)
     Y = _rows_contiguous(expanded.reshape(T * k, N))
     out = torch.empty((T, N), dtype=expanded.dtype, device=expanded.device)
-    _backend.combine(Y, gates.to(expanded.dtype), out, k)
+    _launch("combine", Y, gates.to(expanded.dtype), out, k)
     return out
 
 
@@ -361,7 +433,7 @@ def gate_grad(expanded, grad_out):
     assert grad_out.shape == (T, N)
     Y = _rows_contiguous(expanded.reshape(T * k, N))
     d_gates = torch.empty((T, k), dtype=expanded.dtype, device=expanded.device)
-    _backend.gate_grad(Y, _rows_contiguous(grad_out), d_gates, k)
+    _launch("gate_grad", Y, _rows_contiguous(grad_out), d_gates, k)
     return d_gates
 
 
@@ -370,7 +442,7 @@ def glu_fwd(pre, act=ACT_SILU):
     assert pre.dim() == 2 and pre.size(1) % 2 == 0
     pre = _rows_contiguous(pre)
     h = torch.empty((pre.size(0), pre.size(1) // 2), dtype=pre.dtype, device=pre.device)
-    _backend.glu_fwd(pre, h, act)
+    _launch("glu_fwd", pre, h, act)
     return h
 
 
@@ -378,7 +450,7 @@ def glu_bwd(pre, dh, act=ACT_SILU):
     pre, dh = _rows_contiguous(pre), _rows_contiguous(dh)
     assert dh.size(0) == pre.size(0) and 2 * dh.size(1) == pre.size(1)
     dpre = torch.empty_like(pre)
-    _backend.glu_bwd(pre, dh, dpre, act)
+    _launch("glu_bwd", pre, dh, dpre, act)
     return dpre
 
 
@@ -392,14 +464,17 @@ def scatter2scatter_glu(X, W, sorted_expert_idxs, sorted_scattered_idxs, k, b=No
     assert W.dim() == 3 and W.size(1) == X.size(1) and W.size(2) % 2 == 0
     assert L == (X.size(0) if x_grouped else X.size(0) * k)
     F = W.size(2) // 2
-    if (X.is_cuda and X.dtype in (torch.bfloat16, torch.float16) and not torch.compiler.is_compiling()
-            and hasattr(_backend, "s2s_glu")):
+    if X.is_cuda and X.dtype in (torch.bfloat16, torch.float16) and hasattr(_backend, "s2s_glu"):
         _same_dtype("scatter2scatter_glu", X, W, b)
         off = expert_offsets if expert_offsets is not None else offsets_from_sorted(sorted_expert_idxs, W.size(0))
         pre = torch.empty((L, 2 * F), device=X.device, dtype=X.dtype) if need_pre else None
         h = torch.empty((L, F), device=X.device, dtype=X.dtype)
-        if _backend.s2s_glu(_rows_contiguous(X), W, b, pre, h, _as_i64(sorted_expert_idxs),
-                            _as_i64(sorted_scattered_idxs), _as_i64(off), k, x_grouped, act):
+        args = (_rows_contiguous(X), W, b, pre, h, _as_i64(sorted_expert_idxs), _as_i64(sorted_scattered_idxs),
+                _as_i64(off), k, x_grouped, act)
+        if torch.compiler.is_compiling():
+            _s2s_glu_op(*args)               # falls back to the two launches by itself
+            return pre, h
+        if _backend.s2s_glu(*args):
             return pre, h
     pre = scatter2scatter(X, W, sorted_expert_idxs, sorted_scattered_idxs, k, b=b, x_grouped=x_grouped,
                           y_grouped=True, expert_offsets=expert_offsets)
@@ -412,14 +487,17 @@ def scatter2scatter_glu_bwd(DY, W, pre, sorted_expert_idxs, sorted_scattered_idx
     saved pre-activation: glu_bwd(pre, scatter2scatter(DY, W, grouped in and out)) in one launch where possible."""
     L = sorted_expert_idxs.size(0)
     assert DY.size(0) == L and pre.size(0) == L and pre.size(1) == 2 * W.size(2) and W.size(1) == DY.size(1)
-    if (DY.is_cuda and DY.dtype in (torch.bfloat16, torch.float16) and not torch.compiler.is_compiling()
-            and hasattr(_backend, "s2s_glu_bwd")):
+    if DY.is_cuda and DY.dtype in (torch.bfloat16, torch.float16) and hasattr(_backend, "s2s_glu_bwd"):
         _same_dtype("scatter2scatter_glu_bwd", DY, W, pre)
         off = expert_offsets if expert_offsets is not None else offsets_from_sorted(sorted_expert_idxs, W.size(0))
         pre_c = _rows_contiguous(pre)
         dpre = torch.empty_like(pre_c)
-        if _backend.s2s_glu_bwd(_rows_contiguous(DY), W, pre_c, dpre, _as_i64(sorted_expert_idxs),
-                                _as_i64(sorted_scattered_idxs), _as_i64(off), act):
+        args = (_rows_contiguous(DY), W, pre_c, dpre, _as_i64(sorted_expert_idxs), _as_i64(sorted_scattered_idxs),
+                _as_i64(off), act)
+        if torch.compiler.is_compiling():
+            _s2s_glu_bwd_op(*args)
+            return dpre
+        if _backend.s2s_glu_bwd(*args):
             return dpre
     dh = scatter2scatter(DY, W, sorted_expert_idxs, sorted_scattered_idxs, 1, x_grouped=True, y_grouped=True,
                          expert_offsets=expert_offsets)
@@ -435,7 +513,7 @@ class _TopkSoftmax(torch.autograd.Function):
         T, E = logits.shape
         weights = torch.empty((T, k), dtype=torch.float32, device=logits.device)
         experts = torch.empty((T, k), dtype=torch.int64, device=logits.device)
-        _backend.topk_softmax(logits, weights, experts, renormalize)
+        _launch("topk_softmax", logits, weights, experts, renormalize)
         ctx.save_for_backward(logits, weights, experts)
         ctx.renormalize = renormalize
         ctx.mark_non_differentiable(experts)

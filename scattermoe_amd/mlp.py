@@ -135,7 +135,7 @@ class GLUMLP(_SparseMLP):
         return self.activation(gate) * lin
 
     def forward(self, x: torch.Tensor, expert_p: torch.Tensor, expert_idxs: torch.Tensor):
-        if type(self.activation) is not nn.SiLU or torch.compiler.is_compiling():
+        if type(self.activation) is not nn.SiLU:
             return super().forward(x, expert_p, expert_idxs)
         lead = x.shape[:-1]
         tokens = x.view(-1, x.size(-1))

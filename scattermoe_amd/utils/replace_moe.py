@@ -41,7 +41,7 @@ def _is_silu(act_fn):
 def _gated_mlp(tokens, gate_up_w, down_w, k, eid, idx, off, weights, act_fn):
     """Gated expert MLP with `act(gate) * up`, gate = first half of the (E, 2I, H) layer-1 weights.  With SiLU the
     whole block is one autograd node whose GLU rides in the GEMM epilogues; other activations use three nodes."""
-    if _is_silu(act_fn) and tokens.dim() == 2 and not torch.compiler.is_compiling():
+    if _is_silu(act_fn) and tokens.dim() == 2:
         from ..mlp import _GatedMLP
         return _GatedMLP.apply(tokens, gate_up_w, None, down_w, None, weights.to(tokens.dtype), eid, idx, off, k,
                                ops.ACT_SILU_GATE_FIRST)
