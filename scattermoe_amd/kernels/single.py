@@ -2,7 +2,9 @@
 one token (or k already-expanded rows) times the k experts it is routed to.
 
 The reference has a dedicated GEMV kernel that nothing calls; here the call goes through
-`scatter2scatter`, whose small-row tile class streams each routed expert's weights exactly once."""
+`scatter2scatter`, which sends launches of a handful of rows to its own weight-streaming kernels (the row-dot
+kernel for weights with a contiguous contraction axis, ring-buffered 32-row tiles otherwise): each routed
+expert's weights are read exactly once."""
 import torch
 
 from . import ops
