@@ -187,6 +187,25 @@ int smoe_scatter2scatter_glu_bwd(const void* DY, int64_t sdm, int64_t sdk,
                                  int64_t L, int64_t K, int64_t F, int E, int act, int dtype, void* stream);
 
 /*
+ * Decode step of a gated MLP, forward only: OUT[t] = sum_j gates[t,j] * ( W2[e] glu(W1[e] X[t] + b1[e]) + b2[e] ),
+ * e = experts[t,j], for at most 8 (token, slot) rows, in two launches and without a routing triple (every
+ * workgroup orders the handful of expert ids itself).  Replaces GLUMLP.forward (scattermoe/mlp.py:74-95: the
+ * flatten_sort_count of parallel_experts.py:14-21, two scatter2scatter launches, chunk / activation / multiply,
+ * and the gate bmm of parallel_experts.py:38-46) at decode sizes; bit-identical to smoe_route +
+ * smoe_scatter2scatter_glu + smoe_scatter2scatter + smoe_combine on the same inputs.
+ * X (T,d) row stride sxm; experts (T,k) int64 strides set,sek (ids outside [0,E) drop their row); gates (T,k)
+ * strides sgt,sgk; W1 (E,2F,d) strides sw1e,sw1n (d contiguous); W2 (E,d,F) strides sw2e,sw2n (F contiguous);
+ * b1 (E,2F) / b2 (E,d) or NULL; H (T*k,F) row stride shm: workspace for the hidden rows; OUT (T,d) row stride som.
+ * `act` as for smoe_glu_fwd.  Returns SMOE_ERR_UNSUPPORTED (nothing launched) for float32, more than 8 rows, or
+ * operands whose rows are not 16-byte aligned: the caller then issues the general sequence.
+ */
+int smoe_decode_glu_mlp(const void* X, int64_t sxm, const int64_t* experts, int64_t set, int64_t sek, const void* gates,
+                        int64_t sgt, int64_t sgk, const void* W1, int64_t sw1e, int64_t sw1n, const void* b1,
+                        int64_t sb1e, int64_t sb1n, const void* W2, int64_t sw2e, int64_t sw2n, const void* b2,
+                        int64_t sb2e, int64_t sb2n, void* H, int64_t shm, void* OUT, int64_t som, int64_t T, int k,
+                        int64_t d, int64_t F, int E, int act, int dtype, void* stream);
+
+/*
  * Router front end: weights, experts = topk(softmax(logits.float(), -1), k) [; weights /= weights.sum(-1)].
  * Replaces the softmax / topk / renormalise sequence of scattermoe/utils/replace_moe.py:67-71 (the routing of the
  * Hugging Face blocks the reference patches).  logits (T,E) strides slt,sle, dtype `dtype`; weights_out (T,k)

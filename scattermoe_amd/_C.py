@@ -41,6 +41,9 @@ _SIGNATURES = {
                                         _p, _p, _p, _i64, _i64, _i64, _int, _int, _int, _int, _int, _p]),
     "smoe_scatter2scatter_glu_bwd": (_int, [_p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _p, _i64,
                                             _p, _p, _p, _i64, _i64, _i64, _int, _int, _int, _p]),
+    "smoe_decode_glu_mlp": (_int, [_p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64,
+                                   _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _p, _i64, _i64, _int, _i64, _i64,
+                                   _int, _int, _int, _p]),
     "smoe_topk_softmax": (_int, [_p, _i64, _i64, _i64, _int, _int, _int, _p, _i64, _i64, _p, _i64, _i64, _int, _p]),
 }
 

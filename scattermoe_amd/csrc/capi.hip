@@ -194,6 +194,26 @@ int smoe_glu_bwd(const void* pre, int64_t spm, const void* dh, int64_t sdhm, voi
   return launch_glu_bwd(pre, spm, dh, sdhm, dpre, sdpm, rows, (int)f, act, dtype, (hipStream_t)stream);
 }
 
+int smoe_decode_glu_mlp(const void* X, int64_t sxm, const int64_t* experts, int64_t set, int64_t sek, const void* gates,
+                        int64_t sgt, int64_t sgk, const void* W1, int64_t sw1e, int64_t sw1n, const void* b1,
+                        int64_t sb1e, int64_t sb1n, const void* W2, int64_t sw2e, int64_t sw2n, const void* b2,
+                        int64_t sb2e, int64_t sb2n, void* H, int64_t shm, void* OUT, int64_t som, int64_t T, int k,
+                        int64_t d, int64_t F, int E, int act, int dtype, void* stream) {
+  g_err[0] = 0;
+  if (int rc = glu_common_checks("smoe_decode_glu_mlp", T, d, F, E, act, dtype)) return rc;
+  if (k <= 0) { set_error("smoe_decode_glu_mlp: bad top-k"); return SMOE_ERR_SHAPE; }
+  if (T == 0 || d == 0) return 0;
+  if (!X || !experts || !gates || !W1 || !W2 || !H || !OUT) { set_error("smoe_decode_glu_mlp: NULL pointer"); return SMOE_ERR_NULL; }
+  // Not an error: the caller then takes the general path (routing, two scatter2scatter launches, combine)
+  auto al16 = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
+  if (dtype == SMOE_F32 || T * k > DECODE_MAX_ROWS || F == 0 || d % 8 || F % 8 || sxm % 8 || shm % 8 ||
+      sw1e % 8 || sw1n % 8 || sw2e % 8 || sw2n % 8 || !al16(X) || !al16(W1) || !al16(W2) || !al16(H))
+    return SMOE_ERR_UNSUPPORTED;
+  DecodeArgs a{X, sxm, experts, set, sek, gates, sgt, sgk, W1, sw1e, sw1n, b1, sb1e, sb1n, W2, sw2e, sw2n,
+               b2, sb2e, sb2n, H, shm, OUT, som, (int)T, k, (int)d, (int)F, E, act};
+  return launch_decode_glu_mlp(a, dtype, (hipStream_t)stream);
+}
+
 int smoe_topk_softmax(const void* logits, int64_t slt, int64_t sle, int64_t T, int E, int k, int renormalize,
                       float* weights_out, int64_t swt, int64_t swk, int64_t* idx_out, int64_t sit, int64_t sik,
                       int dtype, void* stream) {

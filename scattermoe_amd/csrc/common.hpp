@@ -149,6 +149,22 @@ struct GroupArgs {
   int L, K, fan_out;
 };
 
+// Whole gated MLP for at most DECODE_MAX_ROWS (token, slot) rows, forward only (csrc/s2s_rowdot.hip)
+static constexpr int DECODE_MAX_ROWS = 8;
+struct DecodeArgs {
+  const void* X; int64_t sxm;                        // (T, d) tokens, columns contiguous
+  const int64_t* experts; int64_t set, sek;          // (T, k) expert ids
+  const void* gates; int64_t sgt, sgk;               // (T, k) routing weights
+  const void* W1; int64_t sw1e, sw1n;                // (E, 2F, d), d contiguous
+  const void* b1; int64_t sb1e, sb1n;                // (E, 2F) or NULL
+  const void* W2; int64_t sw2e, sw2n;                // (E, d, F), F contiguous
+  const void* b2; int64_t sb2e, sb2n;                // (E, d) or NULL
+  void* H; int64_t shm;                              // (T*k, F) workspace: hidden rows in slot order
+  void* OUT; int64_t som;                            // (T, d)
+  int T, k, d, F, E, act;
+};
+int launch_decode_glu_mlp(const DecodeArgs& a, int dtype, hipStream_t st);
+
 int launch_s2s_generic(const S2SArgs& a, int dtype, hipStream_t st);
 int launch_xty_generic(const XtYArgs& a, int dtype, hipStream_t st);
 int launch_group(const GroupArgs& a, int dtype, hipStream_t st);

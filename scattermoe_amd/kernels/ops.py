@@ -170,6 +170,27 @@ class HipBackend:
 
 
     @staticmethod
+    def decode_glu_mlp(x, experts, gates, w1, b1, w2, b2, h, out, act):
+        """Whole gated MLP of a decode step; False when the library has no such kernel for this call."""
+        _C.require_gpu(x, "decode_glu_mlp")
+        lib = _C.load()
+        sb1 = (b1.stride(0), b1.stride(1)) if b1 is not None else (0, 0)
+        sb2 = (b2.stride(0), b2.stride(1)) if b2 is not None else (0, 0)
+        with _C.on_device(x.device):
+            rc = lib.smoe_decode_glu_mlp(
+                _C.ptr(x), x.stride(0), _C.ptr(experts), experts.stride(0), experts.stride(1),
+                _C.ptr(gates), gates.stride(0), gates.stride(1),
+                _C.ptr(w1), w1.stride(0), w1.stride(1), _C.ptr(b1), sb1[0], sb1[1],
+                _C.ptr(w2), w2.stride(0), w2.stride(1), _C.ptr(b2), sb2[0], sb2[1],
+                _C.ptr(h), h.stride(0), _C.ptr(out), out.stride(0),
+                x.size(0), experts.size(1), x.size(1), h.size(1), w1.size(0), act,
+                _C.float_code(x.dtype), _C.stream_ptr(x.device))
+        if rc == _C.ERR_UNSUPPORTED:
+            return False
+        _C.check(rc, "smoe_decode_glu_mlp")
+        return True
+
+    @staticmethod
     def topk_softmax(logits, weights, experts, renormalize):
         _C.require_gpu(logits, "topk_softmax")
         lib = _C.load()
@@ -542,3 +563,27 @@ def topk_softmax(router_logits, k, renormalize=True):
     if not 0 < k <= router_logits.size(1):
         raise ValueError("k must be in 1..num_experts")
     return _TopkSoftmax.apply(router_logits, k, renormalize)
+
+
+DECODE_MAX_ROWS = 8
+
+
+def decode_glu_mlp(x, expert_p, expert_idxs, w1, b1, w2, b2, act=ACT_SILU):
+    """Forward of a gated expert MLP for at most DECODE_MAX_ROWS (token, slot) rows in two launches, routing and
+    gate combine included (reference GLUMLP.forward, mlp.py:74-95).  x (T, d), expert_p / expert_idxs (T, k),
+    w1 (E, 2F, d) and w2 (E, d, F) in the ParallelExperts parameter layout.  Returns the (T, d) output, or None
+    when this call is not the kernels' (more rows, float32, CPU tensors, a compiler tracing, unaligned operands):
+    the caller then takes the general path, whose result these kernels reproduce bit for bit."""
+    if (expert_idxs.numel() > DECODE_MAX_ROWS or expert_idxs.numel() == 0 or not x.is_cuda or x.dim() != 2
+            or x.dtype not in (torch.bfloat16, torch.float16) or torch.compiler.is_compiling()
+            or not hasattr(_backend, "decode_glu_mlp")
+            or w1.stride(2) != 1 or w2.stride(2) != 1 or x.stride(1) != 1):
+        return None
+    _same_dtype("decode_glu_mlp", x, w1, w2, b1, b2)
+    T, k = expert_idxs.shape
+    F = w2.size(2)
+    h = torch.empty((T * k, F), dtype=x.dtype, device=x.device)
+    out = torch.empty((T, x.size(1)), dtype=x.dtype, device=x.device)
+    if _backend.decode_glu_mlp(x, _as_i64(expert_idxs), expert_p.to(x.dtype), w1, b1, w2, b2, h, out, act):
+        return out
+    return None

@@ -139,6 +139,11 @@ class GLUMLP(_SparseMLP):
             return super().forward(x, expert_p, expert_idxs)
         lead = x.shape[:-1]
         tokens = x.view(-1, x.size(-1))
+        if expert_idxs.numel() <= ops.DECODE_MAX_ROWS and not torch.is_grad_enabled() and expert_idxs.dim() == 2:
+            out = ops.decode_glu_mlp(tokens, expert_p, expert_idxs, self.experts.weight, self.experts.bias,
+                                     self.output_experts.weight, self.output_experts.bias, ops.ACT_SILU)
+            if out is not None:
+                return out.view(*lead, out.size(-1))
         eid, idx, off = flatten_sort_count(expert_idxs, num_experts=self.num_experts)
         out = _GatedMLP.apply(tokens, self.experts.weight, self.experts.bias, self.output_experts.weight,
                               self.output_experts.bias, expert_p, eid, idx, off, self.top_k, ops.ACT_SILU)

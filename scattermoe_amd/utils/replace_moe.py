@@ -65,6 +65,12 @@ def experts_forward(self, hidden_states, top_k_index, top_k_weights):
     """Drop-in for transformers 5.x `*Experts.forward`: gate_up_proj (E, 2I, H), down_proj (E, H, I),
     `act_fn(gate) * up` with gate = first half; returns (T, H)."""
     k = top_k_index.shape[-1]
+    if (top_k_index.numel() <= ops.DECODE_MAX_ROWS and not torch.is_grad_enabled() and _is_silu(self.act_fn)
+            and hidden_states.dim() == 2 and top_k_index.dim() == 2):
+        out = ops.decode_glu_mlp(hidden_states, top_k_weights, top_k_index, self.gate_up_proj, None, self.down_proj,
+                                 None, ops.ACT_SILU_GATE_FIRST)
+        if out is not None:
+            return out
     eid, idx, off = flatten_sort_count(top_k_index, num_experts=self.num_experts)
     return _gated_mlp(hidden_states, self.gate_up_proj, self.down_proj, k, eid, idx, off, top_k_weights, self.act_fn)
 
