@@ -18,10 +18,13 @@
 //                are used (weight-streaming regime, Mixtral expert shapes with 64..1536 tokens; from there on
 //                the 256x256 two-stage tile)
 //   GM_RING      tile rows that visit a tile column back to back in the ring classes' order (1: -15 %, 4: -4 %)
+//   STRIPE_BELOW average rows per expert under which the 256x256 class uses that order too (Mixtral shape, 1536
+//                tokens: 1.68 -> 1.37 ms for the two forward launches; neutral at 4096, 2 % slower at 8192)
 //   GM_S2S       row super-tiles per raster band of scatter2scatter (4: +3 % on the layer-2 shaped launches)
 //   GM_XTY       the same for groupXtY (unbanded: bands were neutral there)
 static constexpr int ROWS32_BELOW = 24, ROWS64_BELOW = 48, ROWS128_BELOW = 112, ROWS256_BELOW = 224;
 static constexpr int GM_RING = 8;
+static constexpr int STRIPE_BELOW = 1024;
 static constexpr int GM_S2S = 4;
 static constexpr int GM_XTY = 1 << 20;
 #include <type_traits>
@@ -902,7 +905,10 @@ static int launch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
   const int bn = a.glu == 1 ? TL::BN / 2 : TL::BN;     // output columns per tile
   const int n_tiles = (a.N + bn - 1) / bn;
   const int64_t m_tiles = max_tiles(a.L, a.E, TL::BM);
-  const Raster r = TL::NS > 2 ? make_striped(m_tiles, n_tiles, GM_RING) : make_raster(m_tiles, n_tiles, GM_S2S);
+  // With only a few tile rows per expert no weight panel is shared by the tile rows of a super tile; the striped
+  // order at least keeps the tile rows of one expert together on one XCD.
+  const bool striped = TL::NS > 2 || a.L / a.E < STRIPE_BELOW;
+  const Raster r = striped ? make_striped(m_tiles, n_tiles, GM_RING) : make_raster(m_tiles, n_tiles, GM_S2S);
   const int64_t grid = r.grid();
   if (grid > 0x7fffffffLL || m_tiles > 0x7fffffffLL) { set_error("smoe_scatter2scatter: grid too large"); return SMOE_ERR_RANGE; }
   if constexpr (TL::BN % 128 == 0) {
