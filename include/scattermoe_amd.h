@@ -187,6 +187,18 @@ int smoe_scatter2scatter_glu_bwd(const void* DY, int64_t sdm, int64_t sdk,
                                  int64_t L, int64_t K, int64_t F, int E, int act, int dtype, void* stream);
 
 /*
+ * Gated unit of the gpt-oss experts and its gradient, one pass each (scattermoe/utils/replace_moe.py:39-43, five
+ * elementwise torch launches on strided slices there).  pre (rows, 2f), row stride spm, holds (gate, up) pairs in
+ * adjacent columns:  g = min(gate, limit), u = clamp(up, -limit, limit), h[n, c] = (u + 1) * g * sigmoid(alpha * g).
+ * h / dh (rows, f) row strides shm / sdhm; dpre (rows, 2f) row stride sdpm in the layout of pre.  Clamped inputs
+ * receive no gradient (torch.clamp semantics: the bounds themselves still do).
+ */
+int smoe_gpt_oss_glu_fwd(const void* pre, int64_t spm, void* h, int64_t shm, int64_t rows, int64_t f, float alpha,
+                         float limit, int dtype, void* stream);
+int smoe_gpt_oss_glu_bwd(const void* pre, int64_t spm, const void* dh, int64_t sdhm, void* dpre, int64_t sdpm,
+                         int64_t rows, int64_t f, float alpha, float limit, int dtype, void* stream);
+
+/*
  * Decode step of a gated MLP, forward only: OUT[t] = sum_j gates[t,j] * ( W2[e] glu(W1[e] X[t] + b1[e]) + b2[e] ),
  * e = experts[t,j], for at most 8 (token, slot) rows, in two launches and without a routing triple (every
  * workgroup orders the handful of expert ids itself).  Replaces GLUMLP.forward (scattermoe/mlp.py:74-95: the

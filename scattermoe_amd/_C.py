@@ -20,7 +20,7 @@ I64, I32, I16, U8 = 0, 1, 2, 3
 _FLOAT_CODES = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
 _INDEX_CODES = {torch.int64: I64, torch.int32: I32, torch.int16: I16, torch.uint8: U8}
 
-_p, _i64, _int, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t
+_p, _i64, _int, _sz, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_size_t, ctypes.c_float
 
 _SIGNATURES = {
     "smoe_version": (_int, []),
@@ -41,6 +41,8 @@ _SIGNATURES = {
                                         _p, _p, _p, _i64, _i64, _i64, _int, _int, _int, _int, _int, _p]),
     "smoe_scatter2scatter_glu_bwd": (_int, [_p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _p, _i64,
                                             _p, _p, _p, _i64, _i64, _i64, _int, _int, _int, _p]),
+    "smoe_gpt_oss_glu_fwd": (_int, [_p, _i64, _p, _i64, _i64, _i64, _f32, _f32, _int, _p]),
+    "smoe_gpt_oss_glu_bwd": (_int, [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _f32, _f32, _int, _p]),
     "smoe_decode_glu_mlp": (_int, [_p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64,
                                    _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _p, _i64, _i64, _int, _i64, _i64,
                                    _int, _int, _int, _p]),

@@ -194,6 +194,28 @@ int smoe_glu_bwd(const void* pre, int64_t spm, const void* dh, int64_t sdhm, voi
   return launch_glu_bwd(pre, spm, dh, sdhm, dpre, sdpm, rows, (int)f, act, dtype, (hipStream_t)stream);
 }
 
+int smoe_gpt_oss_glu_fwd(const void* pre, int64_t spm, void* h, int64_t shm, int64_t rows, int64_t f, float alpha,
+                         float limit, int dtype, void* stream) {
+  g_err[0] = 0;
+  if (!dtype_ok(dtype)) { set_error("smoe_gpt_oss_glu_fwd: unknown dtype %d", dtype); return SMOE_ERR_DTYPE; }
+  if (rows < 0 || f < 0) { set_error("smoe_gpt_oss_glu_fwd: bad sizes"); return SMOE_ERR_SHAPE; }
+  if (f > 0x3fffffffLL) { set_error("smoe_gpt_oss_glu_fwd: size beyond int32"); return SMOE_ERR_RANGE; }
+  if (rows == 0 || f == 0) return 0;
+  if (!pre || !h) { set_error("smoe_gpt_oss_glu_fwd: NULL pointer"); return SMOE_ERR_NULL; }
+  return launch_oss_glu_fwd(pre, spm, h, shm, rows, (int)f, alpha, limit, dtype, (hipStream_t)stream);
+}
+
+int smoe_gpt_oss_glu_bwd(const void* pre, int64_t spm, const void* dh, int64_t sdhm, void* dpre, int64_t sdpm,
+                         int64_t rows, int64_t f, float alpha, float limit, int dtype, void* stream) {
+  g_err[0] = 0;
+  if (!dtype_ok(dtype)) { set_error("smoe_gpt_oss_glu_bwd: unknown dtype %d", dtype); return SMOE_ERR_DTYPE; }
+  if (rows < 0 || f < 0) { set_error("smoe_gpt_oss_glu_bwd: bad sizes"); return SMOE_ERR_SHAPE; }
+  if (f > 0x3fffffffLL) { set_error("smoe_gpt_oss_glu_bwd: size beyond int32"); return SMOE_ERR_RANGE; }
+  if (rows == 0 || f == 0) return 0;
+  if (!pre || !dh || !dpre) { set_error("smoe_gpt_oss_glu_bwd: NULL pointer"); return SMOE_ERR_NULL; }
+  return launch_oss_glu_bwd(pre, spm, dh, sdhm, dpre, sdpm, rows, (int)f, alpha, limit, dtype, (hipStream_t)stream);
+}
+
 int smoe_decode_glu_mlp(const void* X, int64_t sxm, const int64_t* experts, int64_t set, int64_t sek, const void* gates,
                         int64_t sgt, int64_t sgk, const void* W1, int64_t sw1e, int64_t sw1n, const void* b1,
                         int64_t sb1e, int64_t sb1n, const void* W2, int64_t sw2e, int64_t sw2n, const void* b2,

@@ -182,6 +182,10 @@ int launch_glu_fwd(const void* pre, int64_t sp, void* h, int64_t sh, int64_t row
 int launch_glu_bwd(const void* pre, int64_t sp, const void* dh, int64_t sdh, void* dpre, int64_t sdp, int64_t rows,
                    int f, int act, int dtype, hipStream_t st);
 
+int launch_oss_glu_fwd(const void* pre, int64_t sp, void* h, int64_t sh, int64_t rows, int f, float alpha, float limit,
+                       int dtype, hipStream_t st);
+int launch_oss_glu_bwd(const void* pre, int64_t sp, const void* dh, int64_t sdh, void* dpre, int64_t sdp, int64_t rows,
+                       int f, float alpha, float limit, int dtype, hipStream_t st);
 int launch_topk_softmax(const void* logits, int64_t slt, int64_t sle, float* w, int64_t swt, int64_t swk,
                         int64_t* idx, int64_t sit, int64_t sik, int64_t Tn, int E, int k, int renorm, int dtype,
                         hipStream_t st);

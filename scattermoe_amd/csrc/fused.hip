@@ -134,6 +134,75 @@ __global__ __launch_bounds__(256) void glu_bwd_kernel(const T* __restrict__ pre,
   }
 }
 
+// ---- gpt-oss gated unit ------------------------------------------------------------------------------------
+// pre (rows, 2f) holds (gate, up) pairs in adjacent columns:
+//   g = min(gate, limit); u = clamp(up, -limit, limit); h = (u + 1) * g * sigmoid(alpha * g)
+// (scattermoe/utils/replace_moe.py:39-43).  One pass each way; clamped inputs pass no gradient, as with torch.clamp
+// (the bounds themselves still do).
+__device__ __forceinline__ float oss_h(float gate, float up, float alpha, float limit) {
+  const float g = fminf(gate, limit), u = fminf(fmaxf(up, -limit), limit);
+  return (u + 1.0f) * (g * sigmoidf_(alpha * g));
+}
+__device__ __forceinline__ void oss_grad(float gate, float up, float dh, float alpha, float limit, float& dgate,
+                                         float& dup) {
+  const float g = fminf(gate, limit), u = fminf(fmaxf(up, -limit), limit);
+  const float s = sigmoidf_(alpha * g);
+  const float glu = g * s;
+  dup = (up >= -limit && up <= limit) ? dh * glu : 0.0f;
+  const float dglu = dh * (u + 1.0f);
+  dgate = gate <= limit ? dglu * (s + alpha * g * s * (1.0f - s)) : 0.0f;
+}
+
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void oss_glu_fwd_kernel(const T* __restrict__ pre, int64_t sp, T* __restrict__ h,
+                                                         int64_t sh, int64_t rows, int f, float alpha, float limit) {
+  constexpr int W = VEC ? Pack<T>::n / 2 : 1;            // hidden columns per thread and step
+  const int64_t per_row = f / W, total = rows * per_row;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / per_row, c = (i % per_row) * W;
+    if (VEC) {
+      struct Half { T v[W]; };
+      const Pack<T> p = *(const Pack<T>*)(pre + r * sp + 2 * c);
+      Half o;
+#pragma unroll
+      for (int q = 0; q < W; ++q) o.v[q] = from_f32<T>(oss_h(to_f32(p.v[2 * q]), to_f32(p.v[2 * q + 1]), alpha, limit));
+      *(Half*)(h + r * sh + c) = o;
+    } else {
+      h[r * sh + c] = from_f32<T>(oss_h(to_f32(pre[r * sp + 2 * c]), to_f32(pre[r * sp + 2 * c + 1]), alpha, limit));
+    }
+  }
+}
+
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void oss_glu_bwd_kernel(const T* __restrict__ pre, int64_t sp, const T* __restrict__ dh,
+                                                         int64_t sdh, T* __restrict__ dpre, int64_t sdp, int64_t rows,
+                                                         int f, float alpha, float limit) {
+  constexpr int W = VEC ? Pack<T>::n / 2 : 1;
+  const int64_t per_row = f / W, total = rows * per_row;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / per_row, c = (i % per_row) * W;
+    if (VEC) {
+      struct Half { T v[W]; };
+      const Pack<T> p = *(const Pack<T>*)(pre + r * sp + 2 * c);
+      const Half d = *(const Half*)(dh + r * sdh + c);
+      Pack<T> o;
+#pragma unroll
+      for (int q = 0; q < W; ++q) {
+        float dg, du;
+        oss_grad(to_f32(p.v[2 * q]), to_f32(p.v[2 * q + 1]), to_f32(d.v[q]), alpha, limit, dg, du);
+        o.v[2 * q] = from_f32<T>(dg);
+        o.v[2 * q + 1] = from_f32<T>(du);
+      }
+      *(Pack<T>*)(dpre + r * sdp + 2 * c) = o;
+    } else {
+      float dg, du;
+      oss_grad(to_f32(pre[r * sp + 2 * c]), to_f32(pre[r * sp + 2 * c + 1]), to_f32(dh[r * sdh + c]), alpha, limit, dg, du);
+      dpre[r * sdp + 2 * c] = from_f32<T>(dg);
+      dpre[r * sdp + 2 * c + 1] = from_f32<T>(du);
+    }
+  }
+}
+
 static bool al16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 static unsigned ew_grid(int64_t total) {
   int64_t b = cdiv64(total, 256);
@@ -203,6 +272,38 @@ int launch_glu_fwd(const void* pre, int64_t sp, void* h, int64_t sh, int64_t row
 int launch_glu_bwd(const void* pre, int64_t sp, const void* dh, int64_t sdh, void* dpre, int64_t sdp, int64_t rows,
                    int f, int act, int dtype, hipStream_t st) {
   SMOE_DISPATCH(dtype, glu_bwd_t<T>(pre, sp, dh, sdh, dpre, sdp, rows, f, act, st));
+}
+
+template <typename T>
+static int oss_glu_fwd_t(const void* pre, int64_t sp, void* h, int64_t sh, int64_t rows, int f, float alpha,
+                         float limit, hipStream_t st) {
+  constexpr int vn = 16 / sizeof(T);
+  const bool vec = f % (vn / 2) == 0 && sp % vn == 0 && sh % (vn / 2) == 0 && al16(pre) && ((uintptr_t)h & 7) == 0;
+  const int64_t total = rows * (f / (vec ? vn / 2 : 1));
+  if (vec) hipLaunchKernelGGL((oss_glu_fwd_kernel<T, true>), dim3(ew_grid(total)), dim3(256), 0, st, (const T*)pre, sp, (T*)h, sh, rows, f, alpha, limit);
+  else hipLaunchKernelGGL((oss_glu_fwd_kernel<T, false>), dim3(ew_grid(total)), dim3(256), 0, st, (const T*)pre, sp, (T*)h, sh, rows, f, alpha, limit);
+  return launch_status("oss_glu_fwd_kernel");
+}
+
+template <typename T>
+static int oss_glu_bwd_t(const void* pre, int64_t sp, const void* dh, int64_t sdh, void* dpre, int64_t sdp, int64_t rows,
+                         int f, float alpha, float limit, hipStream_t st) {
+  constexpr int vn = 16 / sizeof(T);
+  const bool vec = f % (vn / 2) == 0 && sp % vn == 0 && sdp % vn == 0 && sdh % (vn / 2) == 0 && al16(pre) && al16(dpre) &&
+                   ((uintptr_t)dh & 7) == 0;
+  const int64_t total = rows * (f / (vec ? vn / 2 : 1));
+  if (vec) hipLaunchKernelGGL((oss_glu_bwd_kernel<T, true>), dim3(ew_grid(total)), dim3(256), 0, st, (const T*)pre, sp, (const T*)dh, sdh, (T*)dpre, sdp, rows, f, alpha, limit);
+  else hipLaunchKernelGGL((oss_glu_bwd_kernel<T, false>), dim3(ew_grid(total)), dim3(256), 0, st, (const T*)pre, sp, (const T*)dh, sdh, (T*)dpre, sdp, rows, f, alpha, limit);
+  return launch_status("oss_glu_bwd_kernel");
+}
+
+int launch_oss_glu_fwd(const void* pre, int64_t sp, void* h, int64_t sh, int64_t rows, int f, float alpha, float limit,
+                       int dtype, hipStream_t st) {
+  SMOE_DISPATCH(dtype, oss_glu_fwd_t<T>(pre, sp, h, sh, rows, f, alpha, limit, st));
+}
+int launch_oss_glu_bwd(const void* pre, int64_t sp, const void* dh, int64_t sdh, void* dpre, int64_t sdp, int64_t rows,
+                       int f, float alpha, float limit, int dtype, hipStream_t st) {
+  SMOE_DISPATCH(dtype, oss_glu_bwd_t<T>(pre, sp, dh, sdh, dpre, sdp, rows, f, alpha, limit, st));
 }
 
 }  // namespace smoe

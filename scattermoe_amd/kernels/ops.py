@@ -170,6 +170,25 @@ class HipBackend:
 
 
     @staticmethod
+    def oss_glu_fwd(pre, h, alpha, limit):
+        _C.require_gpu(pre, "gpt_oss_glu")
+        lib = _C.load()
+        with _C.on_device(pre.device):
+            rc = lib.smoe_gpt_oss_glu_fwd(_C.ptr(pre), pre.stride(0), _C.ptr(h), h.stride(0), pre.size(0), h.size(1),
+                                          alpha, limit, _C.float_code(pre.dtype), _C.stream_ptr(pre.device))
+        _C.check(rc, "smoe_gpt_oss_glu_fwd")
+
+    @staticmethod
+    def oss_glu_bwd(pre, dh, dpre, alpha, limit):
+        _C.require_gpu(pre, "gpt_oss_glu backward")
+        lib = _C.load()
+        with _C.on_device(pre.device):
+            rc = lib.smoe_gpt_oss_glu_bwd(_C.ptr(pre), pre.stride(0), _C.ptr(dh), dh.stride(0), _C.ptr(dpre),
+                                          dpre.stride(0), pre.size(0), dh.size(1), alpha, limit,
+                                          _C.float_code(pre.dtype), _C.stream_ptr(pre.device))
+        _C.check(rc, "smoe_gpt_oss_glu_bwd")
+
+    @staticmethod
     def decode_glu_mlp(x, experts, gates, w1, b1, w2, b2, h, out, act):
         """Whole gated MLP of a decode step; False when the library has no such kernel for this call."""
         _C.require_gpu(x, "decode_glu_mlp")
@@ -242,6 +261,16 @@ def _glu_bwd_op(pre: torch.Tensor, dh: torch.Tensor, dpre: torch.Tensor, act: in
     _backend.glu_bwd(pre, dh, dpre, act)
 
 
+@torch.library.custom_op("scattermoe::gpt_oss_glu_fwd", mutates_args={"h"})
+def _oss_glu_fwd_op(pre: torch.Tensor, h: torch.Tensor, alpha: float, limit: float) -> None:
+    _backend.oss_glu_fwd(pre, h, alpha, limit)
+
+
+@torch.library.custom_op("scattermoe::gpt_oss_glu_bwd", mutates_args={"dpre"})
+def _oss_glu_bwd_op(pre: torch.Tensor, dh: torch.Tensor, dpre: torch.Tensor, alpha: float, limit: float) -> None:
+    _backend.oss_glu_bwd(pre, dh, dpre, alpha, limit)
+
+
 @torch.library.custom_op("scattermoe::topk_softmax", mutates_args={"weights", "experts"})
 def _topk_softmax_op(logits: torch.Tensor, weights: torch.Tensor, experts: torch.Tensor,
                      renormalize: bool) -> None:
@@ -268,7 +297,8 @@ def _s2s_glu_bwd_op(DY: torch.Tensor, W: torch.Tensor, pre: torch.Tensor, dpre: 
 
 
 _COMPILED_OPS = {"route": _route_op, "offsets": _offsets_op, "combine": _combine_op, "gate_grad": _gate_grad_op,
-                 "glu_fwd": _glu_fwd_op, "glu_bwd": _glu_bwd_op, "topk_softmax": _topk_softmax_op}
+                 "glu_fwd": _glu_fwd_op, "glu_bwd": _glu_bwd_op, "topk_softmax": _topk_softmax_op,
+                 "oss_glu_fwd": _oss_glu_fwd_op, "oss_glu_bwd": _oss_glu_bwd_op}
 
 
 def _launch(name, *args):
@@ -362,16 +392,20 @@ def scatter2scatter_compileable(
 # ------------------------------------------------------------------------------------------------
 # groupXtY
 # ------------------------------------------------------------------------------------------------
-def group_bwd_W(DY, X, expert_offsets, E, has_bias=False):
+def group_bwd_W(DY, X, expert_offsets, E, has_bias=False, like=None):
     """Per-expert dW / db over expert-grouped rows (reference ops.py:191-199).
 
-    The returned DW is an (E, K, N) view of a contiguous (E, N, K) buffer, so that after autograd undoes
-    the `weight.permute(0, 2, 1)` of ParallelExperts the parameter gradient is contiguous.  The kernel
-    writes every element (zeros for experts without rows), hence `empty` rather than `zeros`.
+    The returned DW is (E, K, N).  By default it is a view of a contiguous (E, N, K) buffer, so that after autograd
+    undoes the `weight.permute(0, 2, 1)` of ParallelExperts the parameter gradient is contiguous.  `like` (the
+    (E, K, N) weight the gradient belongs to) overrides that: a weight stored with N contiguous (the gpt-oss
+    parameters) gets a gradient stored the same way, so that accumulating it into `.grad` is not a transposing
+    copy of the whole tensor.  The kernel writes every element (zeros for experts without rows), hence `empty`.
     """
     N, K = DY.size(-1), X.size(-1)
-    DWt = torch.empty((E, N, K), device=DY.device, dtype=DY.dtype)
-    DW = DWt.permute(0, 2, 1)
+    if like is not None and like.dim() == 3 and like.stride(2) == 1 and like.stride(1) != 1:
+        DW = torch.empty((E, K, N), device=DY.device, dtype=DY.dtype)
+    else:
+        DW = torch.empty((E, N, K), device=DY.device, dtype=DY.dtype).permute(0, 2, 1)
     Db = torch.empty((E, N), device=DY.device, dtype=DY.dtype) if has_bias else None
     if torch.compiler.is_compiling():
         groupXtY_compileable(E, DW, Db, DY, X, expert_offsets)
@@ -473,6 +507,35 @@ def glu_bwd(pre, dh, act=ACT_SILU):
     dpre = torch.empty_like(pre)
     _launch("glu_bwd", pre, dh, dpre, act)
     return dpre
+
+
+class _GptOssGLU(torch.autograd.Function):
+    """(up + 1) * gate * sigmoid(alpha * gate) over interleaved (gate, up) columns with the clamps of the gpt-oss
+    experts, one pass each way; the pre-activation is saved and the sigmoid recomputed."""
+
+    @staticmethod
+    def forward(ctx, pre, alpha, limit):
+        pre = _rows_contiguous(pre)
+        ctx.save_for_backward(pre)
+        ctx.alpha, ctx.limit = alpha, limit
+        h = torch.empty((pre.size(0), pre.size(1) // 2), dtype=pre.dtype, device=pre.device)
+        _launch("oss_glu_fwd", pre, h, alpha, limit)
+        return h
+
+    @staticmethod
+    def backward(ctx, dh):
+        (pre,) = ctx.saved_tensors
+        dpre = torch.empty_like(pre)
+        _launch("oss_glu_bwd", pre, _rows_contiguous(dh), dpre, ctx.alpha, ctx.limit)
+        return dpre, None, None
+
+
+def gpt_oss_glu(pre, alpha=1.702, limit=7.0):
+    """Hidden layer of the gpt-oss experts from the (rows, 2f) layer-1 output with (gate, up) in adjacent columns
+    (reference replace_moe.py:39-43): gate clamped from above and up clamped to [-limit, limit], then
+    (up + 1) * gate * sigmoid(alpha * gate).  Differentiable."""
+    assert pre.dim() == 2 and pre.size(1) % 2 == 0
+    return _GptOssGLU.apply(pre, float(alpha), float(limit))
 
 
 def scatter2scatter_glu(X, W, sorted_expert_idxs, sorted_scattered_idxs, k, b=None, x_grouped=False,

@@ -97,7 +97,7 @@ class ParallelLinear(torch.autograd.Function):
         if need_w or need_b or (need_x and not grouped_in):
             xg = x if grouped_in else ops.group(x, idx, fan_out=k)
         if need_w or need_b:
-            d_w, d_b = ops.group_bwd_W(DY=dy, X=xg, expert_offsets=off, E=E, has_bias=bias is not None)
+            d_w, d_b = ops.group_bwd_W(DY=dy, X=xg, expert_offsets=off, E=E, has_bias=bias is not None, like=W)
             if not need_w:
                 d_w = None
 

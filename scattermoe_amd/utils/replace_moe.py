@@ -98,10 +98,7 @@ try:
 
         gate_up = parallel_linear(hidden_states, self.gate_up_proj, k, eid, idx, off,
                                   expert_biases=self.gate_up_proj_bias, grouped_in=False, grouped_out=True)
-        gate, up = gate_up[..., ::2], gate_up[..., 1::2]
-        gate = gate.clamp(min=None, max=self.limit)
-        up = up.clamp(min=-self.limit, max=self.limit)
-        hidden = (up + 1) * (gate * torch.sigmoid(gate * self.alpha))
+        hidden = ops.gpt_oss_glu(gate_up, self.alpha, self.limit)      # clamp, sigmoid gate, (up + 1) * glu: one pass
 
         out = parallel_linear(hidden, self.down_proj, 1, eid, idx, off,
                               expert_biases=self.down_proj_bias, grouped_in=True, grouped_out=False,

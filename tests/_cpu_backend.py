@@ -59,3 +59,14 @@ class OracleBackend:
     def topk_softmax(logits, weights, experts, renormalize):
         w, i = oracle.topk_softmax_ref(logits, weights.size(1), renormalize)
         weights.copy_(w); experts.copy_(i)
+
+    @staticmethod
+    def oss_glu_fwd(pre, h, alpha, limit):
+        h.copy_(oracle.gpt_oss_glu(alpha, limit)(pre.float()))
+
+    @staticmethod
+    def oss_glu_bwd(pre, dh, dpre, alpha, limit):
+        with torch.enable_grad():
+            p = pre.detach().float().requires_grad_()
+            (g,) = torch.autograd.grad(oracle.gpt_oss_glu(alpha, limit)(p), p, dh.float())
+        dpre.copy_(g)

@@ -51,6 +51,8 @@ def test_gpt_oss_patched_forward_backward(dtype, rtol, atol):
     _close(got, want, rtol, atol)
     for a, b in zip(gg, gw):
         _close(a, b, rtol, atol)
+    # weight gradients come back in the layout of the (E, in, out) parameters: nothing left to transpose
+    assert gg[2].is_contiguous() and gg[3].is_contiguous()
 
 
 def test_hf_experts_gate_first_glu():

@@ -209,3 +209,28 @@ def test_glu_fwd_bwd(rows, f, dtype):
     dpre = ops.glu_bwd(pre.to(DEV), dh.to(DEV))
     _close(h, h_ref.detach(), dtype, scale=0.1)
     _close(dpre, ref_in.grad, dtype, scale=0.1)
+
+
+# ---------------------------------------------------------------------------------------------------
+# gpt-oss gated unit: one pass each way against the oracle's chain of torch ops (fp32) and its autograd gradient
+# ---------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,f", [(1, 4), (37, 50), (300, 2880), (64, 1001)])
+def test_gpt_oss_glu(rows, f, dtype):
+    g = torch.Generator().manual_seed(rows + f)
+    pre = (torch.randn(rows, 2 * f, generator=g) * 4).to(dtype)      # +-4 sigma: both clamps (limit 7) are hit
+    pre[0, :4] = torch.tensor([7.0, 7.0, 7.0, -7.0]).to(dtype)       # exactly on the bounds: gradient passes
+    dh = torch.randn(rows, f, generator=g).to(dtype)
+    ref_in = pre.float().requires_grad_()
+    want = oracle.gpt_oss_glu(1.702, 7.0)(ref_in)
+    (want_grad,) = torch.autograd.grad(want, ref_in, dh.float())
+    x = pre.to(DEV).detach().requires_grad_()
+    got = ops.gpt_oss_glu(x, 1.702, 7.0)
+    (got_grad,) = torch.autograd.grad(got, x, dh.to(DEV))
+    want = want.detach()
+    _close(got.detach(), want, dtype, scale=max(1.0, float(want.abs().max())))
+    _close(got_grad, want_grad, dtype, scale=max(1.0, float(want_grad.abs().max())))
+    # strided rows (a column slice of a wider buffer)
+    wide = torch.zeros(rows, 2 * f + 6, dtype=dtype, device=DEV)
+    wide[:, :2 * f] = pre.to(DEV)
+    _close(ops.gpt_oss_glu(wide[:, :2 * f], 1.702, 7.0), want, dtype, scale=max(1.0, float(want.abs().max())))
