@@ -844,9 +844,12 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
 
   AOp A;
   A.rot = (n_loc * AOp::R / Raster::SN) % AOp::R;      // the row panel has SN sharers
-  const char* Xb = (const char*)a.X;
+  // Lane offsets are 32-bit: grouped input rows are taken relative to the tile's first row (so that the input may
+  // be of any size), gathered ones relative to the start of the token matrix.
   const int64_t sxm = a.sxm;
-  A.init(Xb, [&](int row) { return (int64_t)sSrc[row] * sxm * 2; });
+  const int src0 = a.x_grouped ? row0 : 0;
+  const char* Xb = (const char*)a.X + (int64_t)src0 * sxm * 2;
+  A.init(Xb, [&](int row) { return (int64_t)(sSrc[row] - src0) * sxm * 2; });
   BOp B;
   B.rot = (m_loc * BOp::R / Raster::SM) % BOp::R;      // the column panel has SM sharers
   const char* Wb = (const char*)a.W + (int64_t)e * a.swe * 2;
@@ -954,7 +957,7 @@ bool try_s2s_mfma(const S2SArgs& a, int dtype, hipStream_t st, int& rc) {
   else if (a.swn == 1 && a.swk % 8 == 0 && a.N % 8 == 0) b_tr = true;
   else return false;
   // lane offsets inside the kernel are 32-bit byte offsets from a scalar base (X, and W[e])
-  const int64_t x_rows = a.x_grouped ? a.L : a.L / a.fan_out;
+  const int64_t x_rows = a.x_grouped ? 256 : a.L / a.fan_out;        // grouped rows: relative to the tile's first row
   if (fits_u32((x_rows - 1) * a.sxm * 2 + (int64_t)a.K * 2) == false) return false;
   const int64_t w_cols = a.glu == 1 ? 2 * (int64_t)a.N : a.N;
   if (b_tr ? !fits_u32(BK * a.swk * 2 + w_cols * 2) : !fits_u32((w_cols - 1) * a.swn * 2 + (int64_t)a.K * 2))

@@ -130,3 +130,29 @@ def test_module_sampled_tokens_against_per_token_oracle(big):
         # abs 1e-2 relative to the magnitude of the output vector, rel 2e-2
         scale = max(1.0, float(want.abs().max()))
         assert bool((err <= 1e-2 * scale + 2e-2 * want.abs()).all()), "token %d max err %g" % (t, float(err.max()))
+
+
+def test_grouped_input_larger_than_4_gib():
+    """An expert-grouped activation matrix beyond 4 GiB (lane offsets inside the MFMA kernels are 32-bit and taken
+    relative to each tile's first row): rows on both sides of the 4 GiB mark against the oracle's row products, and
+    the launch must be fast enough to have been the MFMA kernel (the any-layout path takes seconds here)."""
+    L, Fh, N, En = 160000, 14336, 512, 4                     # 4.59 GB of bf16 hidden rows
+    gd = torch.Generator(device=DEV).manual_seed(5)
+    h = torch.empty(L, Fh, device=DEV, dtype=BF).normal_(generator=gd)
+    w = (torch.randn(En, N, Fh, generator=gd, device=DEV) * 0.02).to(BF)
+    eid = torch.arange(L, device=DEV) * En // L              # already sorted: L / En rows per expert
+    idx = torch.arange(L, device=DEV)
+    off = torch.tensor([(e + 1) * L // En for e in range(En)], device=DEV)
+    y = ops.scatter2scatter(h, w.permute(0, 2, 1), eid, idx, 1, x_grouped=True, y_grouped=True, expert_offsets=off)
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    ops.scatter2scatter(h, w.permute(0, 2, 1), eid, idx, 1, x_grouped=True, y_grouped=True, expert_offsets=off, out=y)
+    b.record()
+    torch.cuda.synchronize()
+    assert a.elapsed_time(b) < 60.0, "%.1f ms: not the MFMA path" % a.elapsed_time(b)     # 2.3e12 FLOP
+    mark = (1 << 32) // (Fh * 2)                             # first row that starts beyond 4 GiB
+    for n in [0, 39999, 40000, mark - 1, mark, mark + 1, 120000, L - 1]:
+        e = int(eid[n])
+        want = h[n].float().cpu() @ w[e].float().cpu().t()
+        _close(y[n], want, Fh)
