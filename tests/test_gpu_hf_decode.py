@@ -79,6 +79,14 @@ def test_hf_experts_gate_first_glu():
     mg.load_state_dict(m.state_dict())
     got = src.experts_forward(mg, x.to(DEV), index.to(DEV), weights.to(DEV))
     _close(got, want, 1e-4, 1e-5)
+    # decode sizes in bf16 without autograd take the two-launch step: same bits as the general path, close to fp32
+    mh = mg.to(torch.bfloat16)
+    xs, ws, ix = x[:3].to(DEV).bfloat16(), weights[:3].to(DEV).bfloat16(), index[:3].to(DEV)
+    general = src.experts_forward(mh, xs, ix, ws)
+    with torch.no_grad():
+        step = src.experts_forward(mh, xs, ix, ws)
+    assert torch.equal(step, general.detach())
+    _close(step, want[:3], 3e-2, 2e-2)
 
 
 @pytest.mark.parametrize("T", [1, 8, 64, 256])
