@@ -170,6 +170,8 @@ int launch_xty_generic(const XtYArgs& a, int dtype, hipStream_t st);
 int launch_group(const GroupArgs& a, int dtype, hipStream_t st);
 // MFMA paths return 1 if they took the call, 0 if the shape/layout is not theirs, <0 / >1 never.
 bool try_s2s_mfma(const S2SArgs& a, int dtype, hipStream_t st, int& rc);
+bool try_s2s_f32(const S2SArgs& a, hipStream_t st, int& rc);     // float32 MFMA paths (csrc/gemm_f32.hip)
+bool try_xty_f32(const XtYArgs& a, hipStream_t st, int& rc);
 bool try_s2s_rowdot(const S2SArgs& a, int dtype, hipStream_t st, int& rc);   // few-row launches; after try_s2s_mfma's checks
 bool try_xty_mfma(const XtYArgs& a, int dtype, hipStream_t st, int& rc);
 

@@ -947,6 +947,7 @@ static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 static bool fits_u32(int64_t bytes) { return bytes >= 0 && bytes < (int64_t)0xfff00000LL; }
 
 bool try_s2s_mfma(const S2SArgs& a, int dtype, hipStream_t st, int& rc) {
+  if (dtype == SMOE_F32) return try_s2s_f32(a, st, rc);
   if (dtype != SMOE_BF16 && dtype != SMOE_F16) return false;
   if (a.K < 8 || a.K % 8 != 0) return false;
   if (a.sxk != 1 || a.sxm % 8 != 0 || !aligned16(a.X)) return false;
@@ -1088,6 +1089,7 @@ static int launch_xty(const XtYArgs& a, hipStream_t st) {
 }
 
 bool try_xty_mfma(const XtYArgs& a, int dtype, hipStream_t st, int& rc) {
+  if (dtype == SMOE_F32) return try_xty_f32(a, st, rc);
   if (dtype != SMOE_BF16 && dtype != SMOE_F16) return false;
   if (a.K % 8 != 0 || a.N % 8 != 0) return false;
   if (a.sdyn != 1 || a.sxk != 1 || a.sdym % 8 != 0 || a.sxm % 8 != 0) return false;

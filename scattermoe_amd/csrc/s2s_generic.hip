@@ -1,7 +1,7 @@
 // scatter2scatter, layout-agnostic path: any dtype (fp32 / bf16 / fp16), any strides, any sizes.
 // Counterpart of _scatter2scatter (scattermoe/kernels/ops.py:50-118, inner loop :11-42).
 // 64x64 output tiles that never straddle experts, fp32 FMA accumulation through LDS tiles.
-// This is the exact-fp32 path (gfx950 has no TF32) and the fallback for shapes the MFMA path declines.
+// This is the fallback for the shapes and layouts the MFMA paths (bf16 / fp16 / fp32) decline.
 #include "common.hpp"
 
 namespace smoe {
