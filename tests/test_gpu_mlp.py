@@ -112,3 +112,39 @@ def test_empty_batch(cls, dtype):
     assert x.grad.shape == (0, 64) and p.grad.shape == (0, 2)
     for prm in m.parameters():
         assert prm.grad is not None and not prm.grad.isnan().any() and float(prm.grad.abs().max()) == 0.0
+
+
+def _random_module_cases():
+    import random
+    rnd = random.Random(7)
+    out = []
+    for rows_per_expert in (0.5, 3, 20, 30, 60, 100, 150, 260, 400):
+        E = rnd.choice((4, 8, 8, 24))
+        k = min(rnd.choice((1, 2, 2, 4)), E)
+        T = max(1, round(rows_per_expert * E / k))
+        d = rnd.choice((64, 136, 256, 520))
+        f = rnd.choice((40, 128, 264, 512))
+        out.append((T, E, k, d, f, rnd.choice(("glu", "mlp")), rnd.random() < 0.5,
+                    rnd.choice((torch.bfloat16, torch.float16, torch.float32)), rnd.random() < 0.4))
+    return out
+
+
+@pytest.mark.parametrize("T,E,k,d,f,kind,bias,dtype,skew", _random_module_cases())
+def test_module_random_shapes(T, E, k, d, f, kind, bias, dtype, skew):
+    """Forward and every gradient of MLP / GLUMLP at seeded random sizes that cross the tile-class thresholds,
+    against the oracle's per-expert form differentiated by autograd."""
+    g = torch.Generator().manual_seed(T * 31 + d)
+    logits = torch.randn(T, E, generator=g)
+    if skew:
+        logits = logits - 1.5 * torch.log(torch.arange(1, E + 1, dtype=torch.float32))
+    p, experts = torch.topk(torch.softmax(logits, -1), k)
+    x = torch.randn(T, d, generator=g)
+    dy = torch.randn(T, d, generator=g)
+    torch.manual_seed(d + f)
+    m = (GLUMLP(d, f, E, k, bias=bias) if kind == "glu" else MLP(d, f, E, k, bias=bias, activation=nn.GELU()))
+    with torch.no_grad():
+        for prm in m.parameters():
+            prm.normal_(0, 0.05)
+    rtol, atol = (1e-4, 1e-5) if dtype == torch.float32 else (2e-2, 1e-2)
+    for n, a, b in _run_pair(m, x, p, experts, dy, dtype):
+        _rel_check(n, a, b, rtol, atol)
