@@ -5,7 +5,6 @@ The reference has a dedicated GEMV kernel that nothing calls; here the call goes
 `scatter2scatter`, which sends launches of a handful of rows to its own weight-streaming kernels (the row-dot
 kernel for weights with a contiguous contraction axis, ring-buffered 32-row tiles otherwise): each routed
 expert's weights are read exactly once."""
-import torch
 
 from . import ops
 

@@ -1,6 +1,5 @@
 """Seeded synthetic inputs for the benchmark configurations (generated on CPU in fp32, then cast/moved,
 so CPU and GPU runs see identical values).  Draw order: router logits, X, W1, W2, [b1, b2], dY."""
-import math
 from dataclasses import dataclass
 
 import torch
