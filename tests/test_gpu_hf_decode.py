@@ -155,3 +155,40 @@ def test_decode_forward_replays_from_a_hip_graph(T):
             want = step(x, logits)                       # eager work between the replays
             torch.cuda.synchronize()
             assert torch.equal(got, want), "replay %d differs from the eager result" % r
+
+
+def test_tiny_mixtral_model_end_to_end():
+    """A whole (tiny, randomly initialised) Hugging Face Mixtral with its experts class patched: logits and the
+    gradient of an expert weight against the unpatched model (HF's own per-expert loop), float32."""
+    transformers = pytest.importorskip("transformers")
+    from transformers import MixtralConfig, MixtralForCausalLM
+    import transformers.models.mixtral.modeling_mixtral as MX
+    from scattermoe_amd.utils import replace_moe as src
+    if not hasattr(MX, "MixtralExperts"):
+        pytest.skip("transformers without MixtralExperts")
+    cfg = MixtralConfig(vocab_size=128, hidden_size=64, intermediate_size=96, num_hidden_layers=2,
+                        num_attention_heads=4, num_key_value_heads=2, num_local_experts=4, num_experts_per_tok=2,
+                        max_position_embeddings=64, hidden_act="silu")
+    torch.manual_seed(0)
+    model = MixtralForCausalLM(cfg).to(DEV)
+    ids = torch.randint(0, 128, (2, 17), generator=torch.Generator().manual_seed(1)).to(DEV)
+    original = MX.MixtralExperts.forward
+    try:
+        want = model(ids).logits
+        want.float().pow(2).mean().backward()
+        w_ref = model.model.layers[0].mlp.experts.gate_up_proj.grad.clone()
+        model.zero_grad()
+        src.patch_experts_class(MX.MixtralExperts)
+        got = model(ids).logits
+        assert MX.MixtralExperts.forward is src.experts_forward          # the lazy patch has replaced itself
+        got.float().pow(2).mean().backward()
+        w_got = model.model.layers[0].mlp.experts.gate_up_proj.grad
+        torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-4)
+        torch.testing.assert_close(w_got, w_ref, rtol=1e-3, atol=1e-6)
+        with torch.no_grad():                                            # one new token: the decode step kernels
+            step = model(ids[:, :1]).logits
+        MX.MixtralExperts.forward = original
+        with torch.no_grad():
+            torch.testing.assert_close(step, model(ids[:, :1]).logits, rtol=1e-4, atol=1e-4)
+    finally:
+        MX.MixtralExperts.forward = original
