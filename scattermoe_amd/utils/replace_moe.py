@@ -23,12 +23,15 @@ from ..parallel_experts import flatten_sort_count, parallel_linear
 def replace_function(cls, fun_name):
     """Decorator: install `fun` as `cls.fun_name`, announcing the swap when it is first used."""
     def decorator(fun):
+        fun.__original__ = getattr(cls, fun_name, None)       # what the class had before; kept for comparisons / undo
+
         def first_call(*args, **kwargs):
             logging.info("Replacing `%s.%s` with %s:%s", cls.__name__, fun_name,
                          fun.__code__.co_filename, fun.__name__)
             setattr(cls, fun_name, fun)
             return fun(*args, **kwargs)
         first_call.__wrapped__ = fun
+        first_call.__original__ = fun.__original__
         setattr(cls, fun_name, first_call)
         return fun
     return decorator

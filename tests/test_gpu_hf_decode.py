@@ -192,3 +192,38 @@ def test_tiny_mixtral_model_end_to_end():
             torch.testing.assert_close(step, model(ids[:, :1]).logits, rtol=1e-4, atol=1e-4)
     finally:
         MX.MixtralExperts.forward = original
+
+
+def test_tiny_gpt_oss_model_end_to_end():
+    """A whole tiny gpt-oss with the import-time patch of its experts against the forward the class had before."""
+    transformers = pytest.importorskip("transformers")
+    from transformers import GptOssConfig, GptOssForCausalLM
+    import transformers.models.gpt_oss.modeling_gpt_oss as M
+    from scattermoe_amd.utils import replace_moe as src
+    patched = M.GptOssExperts.forward
+    original = getattr(patched, "__original__", None)
+    if original is None:
+        pytest.skip("GptOssExperts was not patched in this process")
+    cfg = GptOssConfig(vocab_size=128, hidden_size=64, intermediate_size=64, num_hidden_layers=2, head_dim=16,
+                       num_attention_heads=4, num_key_value_heads=2, num_local_experts=4, num_experts_per_tok=2,
+                       max_position_embeddings=64, sliding_window=16, layer_types=["sliding_attention", "full_attention"])
+    torch.manual_seed(0)
+    model = GptOssForCausalLM(cfg).to(DEV)
+    with torch.no_grad():
+        for n, prm in model.named_parameters():
+            if "experts" in n:
+                prm.normal_(0, 0.1)
+    ids = torch.randint(0, 128, (2, 9), generator=torch.Generator().manual_seed(2)).to(DEV)
+    try:
+        got = model(ids).logits
+        got.float().pow(2).mean().backward()
+        g_got = model.model.layers[1].mlp.experts.down_proj.grad.clone()
+        model.zero_grad()
+        M.GptOssExperts.forward = original
+        want = model(ids).logits
+        want.float().pow(2).mean().backward()
+        g_want = model.model.layers[1].mlp.experts.down_proj.grad
+        torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-4)
+        torch.testing.assert_close(g_got, g_want, rtol=1e-3, atol=1e-6)
+    finally:
+        M.GptOssExperts.forward = patched
