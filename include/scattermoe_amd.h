@@ -187,6 +187,22 @@ int smoe_scatter2scatter_glu_bwd(const void* DY, int64_t sdm, int64_t sdk,
                                  int64_t L, int64_t K, int64_t F, int E, int act, int dtype, void* stream);
 
 /*
+ * The same two fusions for the gpt-oss experts (scattermoe/utils/replace_moe.py:31-43 and the layer-2 input
+ * gradient of parallel_experts.py:108-123): W holds 2F columns of (gate, up) pairs, PRE (may be NULL in the forward)
+ * is (L, 2F) in that interleaved layout, H (L, F); alpha / limit as for smoe_gpt_oss_glu_fwd.  bf16 / fp16 only;
+ * SMOE_ERR_UNSUPPORTED where there is no fused kernel (float32, rows that are not 16-byte multiples).
+ */
+int smoe_scatter2scatter_oss_glu(const void* X, int64_t sxm, int64_t sxk, const void* W, int64_t swe, int64_t swk,
+                                 int64_t swn, const void* b, int64_t sbe, int64_t sbn, void* PRE, int64_t spm, void* H,
+                                 int64_t shm, const int64_t* eid, const int64_t* idx, const int64_t* off, int64_t L,
+                                 int64_t K, int64_t F, int E, int fan_out, int x_grouped, float alpha, float limit,
+                                 int dtype, void* stream);
+int smoe_scatter2scatter_oss_glu_bwd(const void* DY, int64_t sdm, int64_t sdk, const void* W, int64_t swe, int64_t swk,
+                                     int64_t swn, const void* PRE, int64_t spm, void* DPRE, int64_t sdpm,
+                                     const int64_t* eid, const int64_t* idx, const int64_t* off, int64_t L, int64_t K,
+                                     int64_t F, int E, float alpha, float limit, int dtype, void* stream);
+
+/*
  * Gated unit of the gpt-oss experts and its gradient, one pass each (scattermoe/utils/replace_moe.py:39-43, five
  * elementwise torch launches on strided slices there).  pre (rows, 2f), row stride spm, holds (gate, up) pairs in
  * adjacent columns:  g = min(gate, limit), u = clamp(up, -limit, limit), h[n, c] = (u + 1) * g * sigmoid(alpha * g).

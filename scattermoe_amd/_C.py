@@ -41,6 +41,10 @@ _SIGNATURES = {
                                         _p, _p, _p, _i64, _i64, _i64, _int, _int, _int, _int, _int, _p]),
     "smoe_scatter2scatter_glu_bwd": (_int, [_p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _p, _i64,
                                             _p, _p, _p, _i64, _i64, _i64, _int, _int, _int, _p]),
+    "smoe_scatter2scatter_oss_glu": (_int, [_p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _i64, _p, _i64, _p, _i64,
+                                            _p, _p, _p, _i64, _i64, _i64, _int, _int, _int, _f32, _f32, _int, _p]),
+    "smoe_scatter2scatter_oss_glu_bwd": (_int, [_p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _p, _i64, _p, _p, _p,
+                                                _i64, _i64, _i64, _int, _f32, _f32, _int, _p]),
     "smoe_gpt_oss_glu_fwd": (_int, [_p, _i64, _p, _i64, _i64, _i64, _f32, _f32, _int, _p]),
     "smoe_gpt_oss_glu_bwd": (_int, [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _f32, _f32, _int, _p]),
     "smoe_decode_glu_mlp": (_int, [_p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64,

@@ -121,6 +121,42 @@ int smoe_scatter2scatter_glu_bwd(const void* DY, int64_t sdm, int64_t sdk, const
   return SMOE_ERR_UNSUPPORTED;
 }
 
+int smoe_scatter2scatter_oss_glu(const void* X, int64_t sxm, int64_t sxk, const void* W, int64_t swe, int64_t swk,
+                                 int64_t swn, const void* b, int64_t sbe, int64_t sbn, void* PRE, int64_t spm, void* H,
+                                 int64_t shm, const int64_t* eid, const int64_t* idx, const int64_t* off, int64_t L,
+                                 int64_t K, int64_t F, int E, int fan_out, int x_grouped, float alpha, float limit,
+                                 int dtype, void* stream) {
+  g_err[0] = 0;
+  if (int rc = glu_common_checks("smoe_scatter2scatter_oss_glu", L, K, F, E, SMOE_ACT_SILU, dtype)) return rc;
+  if (fan_out <= 0) { set_error("smoe_scatter2scatter_oss_glu: bad fan_out"); return SMOE_ERR_SHAPE; }
+  if (L == 0 || F == 0) return 0;
+  if (!X || !W || !H || !idx || !off) { set_error("smoe_scatter2scatter_oss_glu: NULL pointer"); return SMOE_ERR_NULL; }
+  if (dtype == SMOE_F32) return SMOE_ERR_UNSUPPORTED;
+  S2SArgs a{X, sxm, sxk, W, swe, swk, swn, b, sbe, sbn, PRE, spm, 1, eid, idx, off,
+            (int)L, (int)K, (int)(2 * F), E, fan_out, x_grouped, 1};
+  a.glu = 3; a.H = H; a.shm = shm; a.alpha = alpha; a.limit = limit;
+  int rc = 0;
+  if (try_s2s_mfma(a, dtype, (hipStream_t)stream, rc)) return rc;
+  return SMOE_ERR_UNSUPPORTED;
+}
+
+int smoe_scatter2scatter_oss_glu_bwd(const void* DY, int64_t sdm, int64_t sdk, const void* W, int64_t swe, int64_t swk,
+                                     int64_t swn, const void* PRE, int64_t spm, void* DPRE, int64_t sdpm,
+                                     const int64_t* eid, const int64_t* idx, const int64_t* off, int64_t L, int64_t K,
+                                     int64_t F, int E, float alpha, float limit, int dtype, void* stream) {
+  g_err[0] = 0;
+  if (int rc = glu_common_checks("smoe_scatter2scatter_oss_glu_bwd", L, K, F, E, SMOE_ACT_SILU, dtype)) return rc;
+  if (L == 0 || F == 0) return 0;
+  if (!DY || !W || !PRE || !DPRE || !idx || !off) { set_error("smoe_scatter2scatter_oss_glu_bwd: NULL pointer"); return SMOE_ERR_NULL; }
+  if (dtype == SMOE_F32) return SMOE_ERR_UNSUPPORTED;
+  S2SArgs a{DY, sdm, sdk, W, swe, swk, swn, nullptr, 0, 0, DPRE, sdpm, 1, eid, idx, off,
+            (int)L, (int)K, (int)F, E, 1, 1, 1};
+  a.glu = 4; a.aux = PRE; a.saux = spm; a.alpha = alpha; a.limit = limit;
+  int rc = 0;
+  if (try_s2s_mfma(a, dtype, (hipStream_t)stream, rc)) return rc;
+  return SMOE_ERR_UNSUPPORTED;
+}
+
 int smoe_group(const void* A, int64_t sam, int64_t sak, const void* coeff, void* Y, int64_t sym, int64_t syk,
                const int64_t* idx, int64_t L, int64_t K, int fan_out, int dtype, void* stream) {
   g_err[0] = 0;

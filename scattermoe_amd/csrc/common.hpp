@@ -64,6 +64,21 @@ __device__ __forceinline__ float glu_dgat(int act, float dh, float gat, float li
   return t * d;
 }
 
+// gated unit of the gpt-oss experts over one (gate, up) pair and its gradient (clamped inputs pass no gradient)
+__device__ __forceinline__ float oss_h(float gate, float up, float alpha, float limit) {
+  const float g = fminf(gate, limit), u = fminf(fmaxf(up, -limit), limit);
+  return (u + 1.0f) * (g * sigmoidf_(alpha * g));
+}
+__device__ __forceinline__ void oss_grad(float gate, float up, float dh, float alpha, float limit, float& dgate,
+                                         float& dup) {
+  const float g = fminf(gate, limit), u = fminf(fmaxf(up, -limit), limit);
+  const float s = sigmoidf_(alpha * g);
+  const float glu = g * s;
+  dup = (up >= -limit && up <= limit) ? dh * glu : 0.0f;
+  const float dglu = dh * (u + 1.0f);
+  dgate = gate <= limit ? dglu * (s + alpha * g * s * (1.0f - s)) : 0.0f;
+}
+
 // ---- expert-aligned tile lookup -------------------------------------------------------------------
 // Rows are expert-sorted; expert e owns rows [off[e-1], off[e]).  Tiles of height BM never straddle
 // two experts: expert e contributes ceil(count_e / BM) tiles and tiles are numbered expert-major.
@@ -127,9 +142,13 @@ struct S2SArgs {
   // fused gated-linear-unit epilogues (MFMA path only, rows in grouped order):
   //   glu == 1: W has 2N columns; Y (may be NULL) receives the pre-activation (L, 2N), H the hidden (L, N)
   //   glu == 2: Y receives d(pre) (L, 2N) computed from the product (= d hidden) and the saved pre-activation AUX
+  //   glu == 3: gpt-oss form, N = 2F columns holding (gate, up) pairs: Y (may be NULL) receives the pre-activation
+  //             (L, 2F), H the hidden (L, F)
+  //   glu == 4: gpt-oss form, N = F: Y receives d(pre) (L, 2F) from the product (= d hidden) and the saved AUX
   int glu = 0, act = 0;
   const void* aux = nullptr; int64_t saux = 0;
   void* H = nullptr; int64_t shm = 0;
+  float alpha = 0.0f, limit = 0.0f;
 };
 
 struct XtYArgs {

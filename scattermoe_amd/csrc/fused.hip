@@ -139,20 +139,6 @@ __global__ __launch_bounds__(256) void glu_bwd_kernel(const T* __restrict__ pre,
 //   g = min(gate, limit); u = clamp(up, -limit, limit); h = (u + 1) * g * sigmoid(alpha * g)
 // (scattermoe/utils/replace_moe.py:39-43).  One pass each way; clamped inputs pass no gradient, as with torch.clamp
 // (the bounds themselves still do).
-__device__ __forceinline__ float oss_h(float gate, float up, float alpha, float limit) {
-  const float g = fminf(gate, limit), u = fminf(fmaxf(up, -limit), limit);
-  return (u + 1.0f) * (g * sigmoidf_(alpha * g));
-}
-__device__ __forceinline__ void oss_grad(float gate, float up, float dh, float alpha, float limit, float& dgate,
-                                         float& dup) {
-  const float g = fminf(gate, limit), u = fminf(fmaxf(up, -limit), limit);
-  const float s = sigmoidf_(alpha * g);
-  const float glu = g * s;
-  dup = (up >= -limit && up <= limit) ? dh * glu : 0.0f;
-  const float dglu = dh * (u + 1.0f);
-  dgate = gate <= limit ? dglu * (s + alpha * g * s * (1.0f - s)) : 0.0f;
-}
-
 template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void oss_glu_fwd_kernel(const T* __restrict__ pre, int64_t sp, T* __restrict__ h,
                                                          int64_t sh, int64_t rows, int f, float alpha, float limit) {

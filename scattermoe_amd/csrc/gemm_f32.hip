@@ -259,17 +259,25 @@ __global__ __launch_bounds__(FNT) void xty_f32_kernel(XtYPlanF32 a, int p_tiles,
   }
 }
 
-// bias gradient: column sums of dY per expert segment (rows in order, so the sum is deterministic)
+// bias gradient: column sums of dY per expert segment.  A workgroup owns 256 columns of one expert: 64 column threads
+// (16 bytes = 4 columns each) x 4 row lanes; the 4 partial sums of a column are added in a fixed order.
 __global__ __launch_bounds__(256) void colsum_f32_kernel(const float* __restrict__ DY, int64_t ld, int N,
                                                         const int64_t* __restrict__ off, float* __restrict__ Db,
                                                         int64_t sdbe, int64_t sdbn) {
+  __shared__ float part[4][256];
   const int e = blockIdx.y;
-  const int n = blockIdx.x * 256 + threadIdx.x;
-  if (n >= N) return;
+  const int c4 = threadIdx.x & 63, rg = threadIdx.x >> 6;
+  const int n = (blockIdx.x * 64 + c4) * 4;
   const int r_lo = e ? (int)off[e - 1] : 0, r_hi = (int)off[e];
-  float s = 0.0f;
-  for (int r = r_lo; r < r_hi; ++r) s += DY[(int64_t)r * ld + n];
-  Db[(int64_t)e * sdbe + (int64_t)n * sdbn] = s;
+  f32x4 s = {0.f, 0.f, 0.f, 0.f};
+  if (n < N)
+    for (int r = r_lo + rg; r < r_hi; r += 4) s += *(const f32x4*)(DY + (int64_t)r * ld + n);
+#pragma unroll
+  for (int q = 0; q < 4; ++q) part[rg][c4 * 4 + q] = s[q];
+  __syncthreads();
+  const int col = blockIdx.x * 256 + threadIdx.x;
+  if (col < N) Db[(int64_t)e * sdbe + (int64_t)col * sdbn] = ((part[0][threadIdx.x] + part[1][threadIdx.x]) +
+                                                               part[2][threadIdx.x]) + part[3][threadIdx.x];
 }
 
 bool try_xty_f32(const XtYArgs& a, hipStream_t st, int& rc) {

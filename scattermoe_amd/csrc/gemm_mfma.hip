@@ -736,6 +736,88 @@ __device__ __forceinline__ void epilogue_glu_bwd_staged(const f32x16 (&acc)[TL::
   }
 }
 
+// gpt-oss forward through LDS: the tile holds BN consecutive columns of the pre-activation, i.e. BN/2 (gate, up)
+// pairs per row; per 16-byte piece one LDS read, one 16-byte store of the pre-activation (if wanted) and one
+// 8-byte store of four hidden values.
+template <typename T, class TL>
+__device__ __forceinline__ void epilogue_oss_fwd_staged(const f32x16 (&acc)[TL::FM][TL::FN], const S2SArgs& a,
+                                                        int row0, int rows, int n0, const T* __restrict__ bias,
+                                                        char* lds) {
+  typedef T T8 __attribute__((ext_vector_type(8)));
+  typedef T T4 __attribute__((ext_vector_type(4)));
+  constexpr int CPR = TL::BN / 8, PIECES = TL::BM * CPR, PP = PIECES / TL::NT;
+  static_assert(PIECES % TL::NT == 0, "pieces must divide evenly");
+  stage_accumulators<T, TL>(acc, lds, [&](int tc) {
+    return bias != nullptr && n0 + tc < a.N ? to_f32(bias[(int64_t)(n0 + tc) * a.sbn]) : 0.0f;
+  });
+  T* pre = (T*)a.Y;
+  T* hid = (T*)a.H;
+#pragma unroll
+  for (int q = 0; q < PP; ++q) {
+    const int p = q * TL::NT + threadIdx.x;
+    const int row = p / CPR, c = p % CPR, n = n0 + c * 8;
+    if (row >= rows || n >= a.N) continue;
+    const T8 v = *(const T8*)(lds + staged_addr<TL>(row, c * 8));
+    T4 h;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) h[e] = from_f32<T>(oss_h(to_f32(v[2 * e]), to_f32(v[2 * e + 1]), a.alpha, a.limit));
+    const int64_t r = row0 + row;
+    if (pre != nullptr) *(T8*)(pre + r * a.sym + n) = v;
+    *(T4*)(hid + r * a.shm + n / 2) = h;
+  }
+}
+
+// gpt-oss backward through LDS: d(hidden) tile staged; per piece of 8 hidden columns two 16-byte loads of the saved
+// pre-activation pairs and two 16-byte stores of their gradient.
+template <typename T, class TL>
+__device__ __forceinline__ void epilogue_oss_bwd_staged(const f32x16 (&acc)[TL::FM][TL::FN], const S2SArgs& a,
+                                                        int row0, int rows, int n0, char* lds) {
+  typedef T T8 __attribute__((ext_vector_type(8)));
+  constexpr int CPR = TL::BN / 8, PIECES = TL::BM * CPR, PP = PIECES / TL::NT, GRP = PP < 4 ? PP : 4;
+  static_assert(PIECES % TL::NT == 0 && PP % GRP == 0, "pieces must divide evenly");
+  stage_accumulators<T, TL>(acc, lds, [](int) { return 0.0f; });
+  const int F = a.N;
+  const T* pre = (const T*)a.aux;
+  T* dpre = (T*)a.Y;
+#pragma unroll 1
+  for (int q0 = 0; q0 < PP; q0 += GRP) {
+    T8 p1[GRP], p2[GRP], dh[GRP];
+    bool ok[GRP];
+#pragma unroll
+    for (int u = 0; u < GRP; ++u) {
+      const int p = (q0 + u) * TL::NT + threadIdx.x;
+      const int row = p / CPR, c = p % CPR, n = n0 + c * 8;
+      ok[u] = row < rows && n < F;
+      if (ok[u]) {
+        const T* src = pre + (int64_t)(row0 + row) * a.saux + 2 * n;
+        p1[u] = *(const T8*)src;
+        p2[u] = *(const T8*)(src + 8);
+      }
+      dh[u] = *(const T8*)(lds + staged_addr<TL>(row, c * 8));
+    }
+#pragma unroll
+    for (int u = 0; u < GRP; ++u) {
+      if (!ok[u]) continue;
+      const int p = (q0 + u) * TL::NT + threadIdx.x;
+      const int row = p / CPR, n = n0 + (p % CPR) * 8;
+      T8 o1, o2;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float dg, du;
+        oss_grad(to_f32(p1[u][2 * e]), to_f32(p1[u][2 * e + 1]), to_f32(dh[u][e]), a.alpha, a.limit, dg, du);
+        o1[2 * e] = from_f32<T>(dg);
+        o1[2 * e + 1] = from_f32<T>(du);
+        oss_grad(to_f32(p2[u][2 * e]), to_f32(p2[u][2 * e + 1]), to_f32(dh[u][4 + e]), a.alpha, a.limit, dg, du);
+        o2[2 * e] = from_f32<T>(dg);
+        o2[2 * e + 1] = from_f32<T>(du);
+      }
+      T* dst = dpre + (int64_t)(row0 + row) * a.sym + 2 * n;
+      *(T8*)dst = o1;
+      *(T8*)(dst + 8) = o2;
+    }
+  }
+}
+
 // XCD-aware tile order.  Workgroup ids are dealt round-robin to the 8 XCDs (private L2 each), so the 32
 // workgroups an XCD runs side by side are the ids x, x+8, ..., x+248 of one 256-block; they are mapped to
 // one 8 x 4 "super tile" of output tiles.  Per 64-deep slice that group touches 8 row panels + 4 column
@@ -896,10 +978,14 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
     const bool al16 = ((((uintptr_t)a.Y | (uintptr_t)a.H) & 15) == 0) && ((a.sym | a.shm | a.N) & 7) == 0;
     if (al16) epilogue_glu_fwd_staged<T, TL>(acc, a, row0, rows, n0, bias, lds);
     else epilogue_glu_fwd<T, TL>(acc, a, row0, rows, n0, bias);
-  } else {
+  } else if (a.glu == 2) {
     const bool al16 = ((((uintptr_t)a.aux | (uintptr_t)a.Y) & 15) == 0) && ((a.saux | a.sym | a.N) & 7) == 0;
     if (al16) epilogue_glu_bwd_staged<T, TL>(acc, a, row0, rows, n0, lds);
     else epilogue_glu_bwd<T, TL>(acc, a, row0, rows, n0);
+  } else if (a.glu == 3) {
+    epilogue_oss_fwd_staged<T, TL>(acc, a, row0, rows, n0, bias, lds);      // alignment checked by the launcher
+  } else {
+    epilogue_oss_bwd_staged<T, TL>(acc, a, row0, rows, n0, lds);
   }
 }
 
@@ -926,6 +1012,12 @@ static int launch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
 
 template <typename T>
 static int dispatch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
+  // the gpt-oss epilogues exist only in their LDS-staged form (16-byte pieces)
+  if (a.glu == 3 && !((((uintptr_t)a.Y & 15) | ((uintptr_t)a.H & 7)) == 0 && (a.sym & 7) == 0 && (a.shm & 3) == 0 &&
+                      (a.N & 7) == 0))
+    return SMOE_ERR_UNSUPPORTED;
+  if (a.glu == 4 && !((((uintptr_t)a.aux | (uintptr_t)a.Y) & 15) == 0 && ((a.saux | a.sym | a.N) & 7) == 0))
+    return SMOE_ERR_UNSUPPORTED;
   const int64_t avg = a.L / a.E;
   if (avg >= ROWS256_BELOW) return launch_s2s<T, Tile<256, 256, 2, 4>>(a, b_tr, st);
   // Below that the launch is a stream over the weights: ring-buffered classes, tile height by rows per expert
@@ -1041,18 +1133,37 @@ __global__ __launch_bounds__(TL::NT) void xty_mfma_kernel(XtYPlan a, Raster rast
   }
 }
 
-// Bias gradient when dY is the column operand: plain column sums per expert segment.
+// Bias gradient when dY is the column operand: column sums per expert segment.  A workgroup owns 256 columns of one
+// expert: 32 column threads (16 bytes = 8 columns each) x 8 row lanes; every thread adds up the rows r = lane
+// (mod 8) of the segment, then the 8 partial sums of a column are added in a fixed order (deterministic).
 template <typename T>
 __global__ __launch_bounds__(256) void colsum_kernel(const T* __restrict__ DY, int64_t ld, int N,
                                                     const int64_t* __restrict__ off, T* __restrict__ Db,
                                                     int64_t sdbe, int64_t sdbn) {
+  typedef T T8 __attribute__((ext_vector_type(8)));
+  __shared__ float part[8][256];
   const int e = blockIdx.y;
-  const int n = blockIdx.x * 256 + threadIdx.x;
-  if (n >= N) return;
+  const int c8 = threadIdx.x & 31, rg = threadIdx.x >> 5;
+  const int n = (blockIdx.x * 32 + c8) * 8;
   const int r_lo = e ? (int)off[e - 1] : 0, r_hi = (int)off[e];
-  float s = 0.0f;
-  for (int r = r_lo; r < r_hi; ++r) s += to_f32(DY[(int64_t)r * ld + n]);
-  Db[(int64_t)e * sdbe + (int64_t)n * sdbn] = from_f32<T>(s);
+  float s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if (n < N) {
+    for (int r = r_lo + rg; r < r_hi; r += 8) {
+      const T8 v = *(const T8*)(DY + (int64_t)r * ld + n);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) s[q] += to_f32(v[q]);
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < 8; ++q) part[rg][c8 * 8 + q] = s[q];
+  __syncthreads();
+  const int col = blockIdx.x * 256 + threadIdx.x;
+  if (col < N) {
+    float t = 0.0f;
+#pragma unroll
+    for (int g = 0; g < 8; ++g) t += part[g][threadIdx.x];
+    Db[(int64_t)e * sdbe + (int64_t)col * sdbn] = from_f32<T>(t);
+  }
 }
 
 template <typename T>

@@ -179,7 +179,7 @@ __global__ __launch_bounds__(RD_WAVES * 64) void s2s_rowdot_kernel(S2SArgs a, in
 // Called with the operand checks of the MFMA path already done (K-contiguous weights, 16-byte aligned rows,
 // K a multiple of 8).  Returns false when the shape is not this kernel's.
 bool try_s2s_rowdot(const S2SArgs& a, int dtype, hipStream_t st, int& rc) {
-  if (a.glu == 2 || a.L > ROWDOT_MAX_ROWS) return false;
+  if (a.glu >= 2 || a.L > ROWDOT_MAX_ROWS) return false;
   const int64_t m_tiles = max_tiles(a.L, a.E, RD_R);
   const int n_groups = a.glu == 1 ? (a.N + RD_C / 2 - 1) / (RD_C / 2) : (a.N + RD_C - 1) / RD_C;
   // enough workgroups to give every CU several, few enough that the tile lookup is amortised

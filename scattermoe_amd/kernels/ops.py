@@ -170,6 +170,38 @@ class HipBackend:
 
 
     @staticmethod
+    def s2s_oss_glu(X, W, b, pre, h, eid, idx, off, k, x_grouped, alpha, limit):
+        """Fused layer-1 GEMM + gpt-oss gated unit; False when the library has no fused kernel for this call."""
+        _C.require_gpu(X, "scatter2scatter_glu")
+        lib = _C.load()
+        sbe, sbn = (b.stride(0), b.stride(1)) if b is not None else (0, 0)
+        with _C.on_device(X.device):
+            rc = lib.smoe_scatter2scatter_oss_glu(
+                _C.ptr(X), X.stride(0), X.stride(1), _C.ptr(W), W.stride(0), W.stride(1), W.stride(2),
+                _C.ptr(b), sbe, sbn, _C.ptr(pre), pre.stride(0) if pre is not None else 0, _C.ptr(h), h.stride(0),
+                _C.ptr(eid), _C.ptr(idx), _C.ptr(off), eid.numel(), X.size(1), h.size(1), W.size(0), k,
+                int(bool(x_grouped)), alpha, limit, _C.float_code(X.dtype), _C.stream_ptr(X.device))
+        if rc == _C.ERR_UNSUPPORTED:
+            return False
+        _C.check(rc, "smoe_scatter2scatter_oss_glu")
+        return True
+
+    @staticmethod
+    def s2s_oss_glu_bwd(DY, W, pre, dpre, eid, idx, off, alpha, limit):
+        _C.require_gpu(DY, "scatter2scatter_glu_bwd")
+        lib = _C.load()
+        with _C.on_device(DY.device):
+            rc = lib.smoe_scatter2scatter_oss_glu_bwd(
+                _C.ptr(DY), DY.stride(0), DY.stride(1), _C.ptr(W), W.stride(0), W.stride(1), W.stride(2),
+                _C.ptr(pre), pre.stride(0), _C.ptr(dpre), dpre.stride(0), _C.ptr(eid), _C.ptr(idx), _C.ptr(off),
+                eid.numel(), DY.size(1), W.size(2), W.size(0), alpha, limit, _C.float_code(DY.dtype),
+                _C.stream_ptr(DY.device))
+        if rc == _C.ERR_UNSUPPORTED:
+            return False
+        _C.check(rc, "smoe_scatter2scatter_oss_glu_bwd")
+        return True
+
+    @staticmethod
     def oss_glu_fwd(pre, h, alpha, limit):
         _C.require_gpu(pre, "gpt_oss_glu")
         lib = _C.load()
@@ -465,6 +497,7 @@ def group_compileable(A: torch.Tensor, K: int, N: int, Y: torch.Tensor, coeff: O
 # ------------------------------------------------------------------------------------------------
 ACT_SILU = 0               # h = silu(second half) * first half   (GLUMLP of the reference)
 ACT_SILU_GATE_FIRST = 1    # h = silu(first half) * second half   (Hugging Face `act(gate) * up`)
+ACT_GPT_OSS = 2            # (gate, up) in adjacent columns, clamps, (up + 1) * gate * sigmoid(alpha * gate)
 
 
 def _rows_contiguous(t):
@@ -539,52 +572,67 @@ def gpt_oss_glu(pre, alpha=1.702, limit=7.0):
 
 
 def scatter2scatter_glu(X, W, sorted_expert_idxs, sorted_scattered_idxs, k, b=None, x_grouped=False,
-                        act=ACT_SILU, expert_offsets=None, need_pre=True):
+                        act=ACT_SILU, expert_offsets=None, need_pre=True, alpha=1.702, limit=7.0):
     """Layer 1 of a gated MLP with its GLU: returns (pre, h) with rows in expert-sorted order, where
     pre = scatter2scatter(X, W, ..., y_grouped=True) (L, 2F) and h = glu_fwd(pre) (L, F)
-    (reference mlp.py:74-87).  One fused launch where the library has one, the two calls otherwise (same
-    results up to one unit in the last place of rare elements).  `need_pre=False` (inference) lets the fused launch skip storing `pre`."""
+    (reference mlp.py:74-87; `act=ACT_GPT_OSS`: the gated unit of replace_moe.py:39-43 with `alpha`, `limit`).
+    One fused launch where the library has one, the two calls otherwise (same results up to one unit in the last
+    place of rare elements).  `need_pre=False` (inference) lets the fused launch skip storing `pre`."""
     L = sorted_expert_idxs.size(0)
     assert W.dim() == 3 and W.size(1) == X.size(1) and W.size(2) % 2 == 0
     assert L == (X.size(0) if x_grouped else X.size(0) * k)
     F = W.size(2) // 2
+    oss = act == ACT_GPT_OSS
     if X.is_cuda and X.dtype in (torch.bfloat16, torch.float16) and hasattr(_backend, "s2s_glu"):
         _same_dtype("scatter2scatter_glu", X, W, b)
         off = expert_offsets if expert_offsets is not None else offsets_from_sorted(sorted_expert_idxs, W.size(0))
         pre = torch.empty((L, 2 * F), device=X.device, dtype=X.dtype) if need_pre else None
         h = torch.empty((L, F), device=X.device, dtype=X.dtype)
         args = (_rows_contiguous(X), W, b, pre, h, _as_i64(sorted_expert_idxs), _as_i64(sorted_scattered_idxs),
-                _as_i64(off), k, x_grouped, act)
+                _as_i64(off), k, x_grouped)
         if torch.compiler.is_compiling():
-            _s2s_glu_op(*args)               # falls back to the two launches by itself
-            return pre, h
-        if _backend.s2s_glu(*args):
+            if not oss:
+                _s2s_glu_op(*args, act)          # falls back to the two launches by itself
+                return pre, h
+        elif (_backend.s2s_oss_glu(*args, float(alpha), float(limit)) if oss else _backend.s2s_glu(*args, act)):
             return pre, h
     pre = scatter2scatter(X, W, sorted_expert_idxs, sorted_scattered_idxs, k, b=b, x_grouped=x_grouped,
                           y_grouped=True, expert_offsets=expert_offsets)
+    if oss:
+        h = torch.empty((L, F), dtype=pre.dtype, device=pre.device)
+        _launch("oss_glu_fwd", pre, h, float(alpha), float(limit))
+        return pre, h
     return pre, glu_fwd(pre, act)
 
 
 def scatter2scatter_glu_bwd(DY, W, pre, sorted_expert_idxs, sorted_scattered_idxs, act=ACT_SILU,
-                            expert_offsets=None):
+                            expert_offsets=None, alpha=1.702, limit=7.0):
     """d(pre) (L, 2F) from the grouped output gradient DY (L, K) of layer 2, its weights W (E, K, F) and the
     saved pre-activation: glu_bwd(pre, scatter2scatter(DY, W, grouped in and out)) in one launch where possible."""
     L = sorted_expert_idxs.size(0)
     assert DY.size(0) == L and pre.size(0) == L and pre.size(1) == 2 * W.size(2) and W.size(1) == DY.size(1)
+    oss = act == ACT_GPT_OSS
     if DY.is_cuda and DY.dtype in (torch.bfloat16, torch.float16) and hasattr(_backend, "s2s_glu_bwd"):
         _same_dtype("scatter2scatter_glu_bwd", DY, W, pre)
         off = expert_offsets if expert_offsets is not None else offsets_from_sorted(sorted_expert_idxs, W.size(0))
         pre_c = _rows_contiguous(pre)
         dpre = torch.empty_like(pre_c)
         args = (_rows_contiguous(DY), W, pre_c, dpre, _as_i64(sorted_expert_idxs), _as_i64(sorted_scattered_idxs),
-                _as_i64(off), act)
+                _as_i64(off))
         if torch.compiler.is_compiling():
-            _s2s_glu_bwd_op(*args)
-            return dpre
-        if _backend.s2s_glu_bwd(*args):
+            if not oss:
+                _s2s_glu_bwd_op(*args, act)
+                return dpre
+        elif (_backend.s2s_oss_glu_bwd(*args, float(alpha), float(limit)) if oss
+              else _backend.s2s_glu_bwd(*args, act)):
             return dpre
     dh = scatter2scatter(DY, W, sorted_expert_idxs, sorted_scattered_idxs, 1, x_grouped=True, y_grouped=True,
                          expert_offsets=expert_offsets)
+    if oss:
+        pre_c = _rows_contiguous(pre)
+        dpre = torch.empty_like(pre_c)
+        _launch("oss_glu_bwd", pre_c, _rows_contiguous(dh), dpre, float(alpha), float(limit))
+        return dpre
     return glu_bwd(pre, dh, act)
 
 

@@ -27,22 +27,26 @@ class _GatedMLP(torch.autograd.Function):
     """The whole gated expert MLP as one autograd node, so that the gated linear unit can ride in the epilogues
     of the GEMMs around it: forward = layer 1 + GLU (one launch), layer 2, gate-weighted combine; backward =
     the dataflow of two chained ParallelLinear nodes (reference parallel_experts.py:64-134) with the layer-2
-    input gradient and the GLU gradient in one launch.  Same numerics as the unfused chain (intermediates are rounded to the storage type at the same points)."""
+    input gradient and the GLU gradient in one launch.  Same numerics as the unfused chain (intermediates are
+    rounded to the storage type at the same points).
+
+    w1 (E, d, 2F) and w2 (E, F, d) are the (E, in, out) views the kernels take, in either memory layout: the
+    permuted ParallelExperts parameters, or weights stored that way (gpt-oss); their gradients come back in the
+    layout of the weight they belong to.  `act`: ops.ACT_SILU / ACT_SILU_GATE_FIRST / ACT_GPT_OSS (+ alpha, limit)."""
 
     @staticmethod
-    def forward(ctx, x, w1, b1, w2, b2, gates, eid, idx, off, k, act):
-        # w1 (E, 2F, d), w2 (E, d, F): the ParallelExperts parameters; the kernels take the (E, in, out) views
+    def forward(ctx, x, w1, b1, w2, b2, gates, eid, idx, off, k, act, alpha=1.702, limit=7.0):
         T = x.size(0)
         need_grad = any(ctx.needs_input_grad[:6])
-        pre, h = ops.scatter2scatter_glu(x, w1.permute(0, 2, 1), eid, idx, k, b=b1, act=act,
-                                         expert_offsets=off, need_pre=need_grad)
-        expanded = ops.scatter2scatter(h, w2.permute(0, 2, 1), eid, idx, 1, b=b2, x_grouped=True,
-                                       y_grouped=False, expert_offsets=off)
+        pre, h = ops.scatter2scatter_glu(x, w1, eid, idx, k, b=b1, act=act, expert_offsets=off,
+                                         need_pre=need_grad, alpha=alpha, limit=limit)
+        expanded = ops.scatter2scatter(h, w2, eid, idx, 1, b=b2, x_grouped=True, y_grouped=False,
+                                       expert_offsets=off)
         kept = expanded.view(T, k, expanded.size(-1))
         out = ops.combine(kept, gates)
         if need_grad:
             ctx.save_for_backward(x, w1, b1, w2, b2, gates, eid, idx, off, pre, h, kept)
-        ctx.k, ctx.act = k, act
+        ctx.k, ctx.act, ctx.alpha, ctx.limit = k, act, alpha, limit
         return out
 
     @staticmethod
@@ -61,21 +65,22 @@ class _GatedMLP(torch.autograd.Function):
                        out=kept.view(-1, kept.size(-1)))
         d_w2 = d_b2 = None
         if need_w2 or need_b2:
-            d_w2, d_b2 = ops.group_bwd_W(DY=dy, X=h, expert_offsets=off, E=E, has_bias=b2 is not None)
-            d_w2 = d_w2.permute(0, 2, 1) if need_w2 else None     # back to the parameter layout (E, d, F)
+            d_w2, d_b2 = ops.group_bwd_W(DY=dy, X=h, expert_offsets=off, E=E, has_bias=b2 is not None, like=w2)
+            d_w2 = d_w2 if need_w2 else None
         d_x = d_w1 = d_b1 = None
         if need_x or need_w1 or need_b1:
-            dpre = ops.scatter2scatter_glu_bwd(dy, w2, pre, eid, idx, act=act, expert_offsets=off)
+            dpre = ops.scatter2scatter_glu_bwd(dy, w2.permute(0, 2, 1), pre, eid, idx, act=act, expert_offsets=off,
+                                               alpha=ctx.alpha, limit=ctx.limit)
             xg = ops.group(x, idx, fan_out=k)
             if need_w1 or need_b1:
-                d_w1, d_b1 = ops.group_bwd_W(DY=dpre, X=xg, expert_offsets=off, E=E, has_bias=b1 is not None)
-                d_w1 = d_w1.permute(0, 2, 1) if need_w1 else None
+                d_w1, d_b1 = ops.group_bwd_W(DY=dpre, X=xg, expert_offsets=off, E=E, has_bias=b1 is not None, like=w1)
+                d_w1 = d_w1 if need_w1 else None
             if need_x:
-                d_exp = ops.scatter2scatter(dpre, w1, eid, idx, 1, x_grouped=True, y_grouped=False,
+                d_exp = ops.scatter2scatter(dpre, w1.permute(0, 2, 1), eid, idx, 1, x_grouped=True, y_grouped=False,
                                             out=xg, expert_offsets=off)
                 d_x = d_exp if k == 1 else d_exp.view(x.size(0), k, d_exp.size(-1)).sum(-2)
         return d_x, d_w1, (d_b1 if need_b1 else None), d_w2, (d_b2 if need_b2 else None), d_gates, \
-            None, None, None, None, None
+            None, None, None, None, None, None, None
 
 
 class _SparseMLP(nn.Module):
@@ -145,6 +150,7 @@ class GLUMLP(_SparseMLP):
             if out is not None:
                 return out.view(*lead, out.size(-1))
         eid, idx, off = flatten_sort_count(expert_idxs, num_experts=self.num_experts)
-        out = _GatedMLP.apply(tokens, self.experts.weight, self.experts.bias, self.output_experts.weight,
-                              self.output_experts.bias, expert_p, eid, idx, off, self.top_k, ops.ACT_SILU)
+        out = _GatedMLP.apply(tokens, self.experts.weight.permute(0, 2, 1), self.experts.bias,
+                              self.output_experts.weight.permute(0, 2, 1), self.output_experts.bias, expert_p,
+                              eid, idx, off, self.top_k, ops.ACT_SILU)
         return out.view(*lead, out.size(-1))

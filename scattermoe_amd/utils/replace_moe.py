@@ -46,8 +46,8 @@ def _gated_mlp(tokens, gate_up_w, down_w, k, eid, idx, off, weights, act_fn):
     whole block is one autograd node whose GLU rides in the GEMM epilogues; other activations use three nodes."""
     if _is_silu(act_fn) and tokens.dim() == 2:
         from ..mlp import _GatedMLP
-        return _GatedMLP.apply(tokens, gate_up_w, None, down_w, None, weights.to(tokens.dtype), eid, idx, off, k,
-                               ops.ACT_SILU_GATE_FIRST)
+        return _GatedMLP.apply(tokens, gate_up_w.permute(0, 2, 1), None, down_w.permute(0, 2, 1), None,
+                               weights.to(tokens.dtype), eid, idx, off, k, ops.ACT_SILU_GATE_FIRST)
     pre = parallel_linear(tokens, gate_up_w.transpose(1, 2), k, eid, idx, off, grouped_in=False, grouped_out=True)
     h = _glu(pre, act_fn, gate_first=True)
     return parallel_linear(h, down_w.transpose(1, 2), 1, eid, idx, off, grouped_in=True, grouped_out=False,
@@ -99,13 +99,19 @@ try:
             routing_weights = torch.gather(routing_weights, dim=1, index=router_indices)
         eid, idx, off = flatten_sort_count(router_indices, num_experts=self.num_experts)
 
-        gate_up = parallel_linear(hidden_states, self.gate_up_proj, k, eid, idx, off,
-                                  expert_biases=self.gate_up_proj_bias, grouped_in=False, grouped_out=True)
-        hidden = ops.gpt_oss_glu(gate_up, self.alpha, self.limit)      # clamp, sigmoid gate, (up + 1) * glu: one pass
-
-        out = parallel_linear(hidden, self.down_proj, 1, eid, idx, off,
-                              expert_biases=self.down_proj_bias, grouped_in=True, grouped_out=False,
-                              gates=routing_weights.to(hidden.dtype))
+        if hidden_states.dtype in (torch.bfloat16, torch.float16) and hidden_states.is_cuda:
+            # one autograd node; the gated unit rides in the epilogues of the GEMMs around it
+            from ..mlp import _GatedMLP
+            out = _GatedMLP.apply(hidden_states, self.gate_up_proj, self.gate_up_proj_bias, self.down_proj,
+                                  self.down_proj_bias, routing_weights.to(hidden_states.dtype), eid, idx, off, k,
+                                  ops.ACT_GPT_OSS, float(self.alpha), float(self.limit))
+        else:
+            gate_up = parallel_linear(hidden_states, self.gate_up_proj, k, eid, idx, off,
+                                      expert_biases=self.gate_up_proj_bias, grouped_in=False, grouped_out=True)
+            hidden = ops.gpt_oss_glu(gate_up, self.alpha, self.limit)      # clamp, sigmoid gate, (up + 1) * glu: one pass
+            out = parallel_linear(hidden, self.down_proj, 1, eid, idx, off,
+                                  expert_biases=self.down_proj_bias, grouped_in=True, grouped_out=False,
+                                  gates=routing_weights.to(hidden.dtype))
         if len(lead_shape) == 3:       # 4.x callers pass (batch, seq, hidden) and expect it back
             return out.view(lead_shape[0], -1, self.hidden_size)
         return out

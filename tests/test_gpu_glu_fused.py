@@ -78,6 +78,47 @@ def test_fused_backward_equals_two_launches(T, E, k, d, F, act, layout, dtype):
     _one_ulp(got, ref)
 
 
+# gpt-oss form: (gate, up) pairs in adjacent columns, weights stored (E, in, out) or transposed
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("layout", ["n_contig", "k_contig"])
+@pytest.mark.parametrize("bias,need_pre", [(True, True), (False, False)])
+@pytest.mark.parametrize("T,E,k,d,F", SHAPES)
+def test_gpt_oss_fused_forward_equals_two_launches(T, E, k, d, F, bias, need_pre, layout, dtype):
+    F = F + (-F) % 4                                   # pairs of pairs: hidden rows must be 8-byte multiples
+    x, w1, b1, eid, idx, off, g = _setup(T, E, k, d, F, dtype)
+    W = w1.permute(0, 2, 1).contiguous() if layout == "n_contig" else w1.permute(0, 2, 1)
+    b = b1 if bias else None
+    pre_ref = ops.scatter2scatter(x, W, eid, idx, k, b=b, y_grouped=True, expert_offsets=off)
+    h_ref = ops.gpt_oss_glu(pre_ref, 1.702, 7.0)
+    pre, h = ops.scatter2scatter_glu(x, W, eid, idx, k, b=b, act=ops.ACT_GPT_OSS, expert_offsets=off,
+                                     need_pre=need_pre, alpha=1.702, limit=7.0)
+    if need_pre:
+        assert torch.equal(pre, pre_ref)
+    _one_ulp(h, h_ref)
+    want = oracle.gpt_oss_glu(1.702, 7.0)(pre_ref.float().cpu())
+    err = (h.float().cpu() - want).abs()
+    assert bool((err <= 1e-2 * max(1.0, float(want.abs().max())) + 2e-2 * want.abs()).all())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("layout", ["n_contig", "k_contig"])
+@pytest.mark.parametrize("T,E,k,d,F", SHAPES)
+def test_gpt_oss_fused_backward_equals_two_launches(T, E, k, d, F, layout, dtype):
+    F = F + (-F) % 8
+    x, w1, b1, eid, idx, off, g = _setup(T, E, k, d, F, dtype)
+    L = T * k
+    w2 = (torch.randn(E, d, F, generator=g) * 0.1).to(dtype).to(DEV)         # (E, K = d, N = F) for the dX product
+    W = w2 if layout == "n_contig" else w2.permute(0, 2, 1).contiguous().permute(0, 2, 1)
+    pre = (torch.randn(L, 2 * F, generator=g) * 4).to(dtype).to(DEV)
+    dy = torch.randn(L, d, generator=g).to(dtype).to(DEV)
+    dh = ops.scatter2scatter(dy, W, eid, idx, 1, x_grouped=True, y_grouped=True, expert_offsets=off)
+    ref = torch.empty_like(pre)
+    ops._launch("oss_glu_bwd", pre, dh, ref, 1.702, 7.0)
+    got = ops.scatter2scatter_glu_bwd(dy, W, pre, eid, idx, act=ops.ACT_GPT_OSS, expert_offsets=off,
+                                      alpha=1.702, limit=7.0)
+    _one_ulp(got, ref)
+
+
 @pytest.mark.parametrize("bias", [False, True])
 @pytest.mark.parametrize("T,E,k,d,F", SHAPES[:5])
 def test_module_matches_unfused_chain(T, E, k, d, F, bias):
