@@ -842,7 +842,11 @@ struct Raster {
       ml = nl = 0;
       return m < m_tiles && n < n_tiles;
     }
-    const int s = (i / (SM * SN)) * 8 + x, r = i % (SM * SN);
+    // The 8 supers of step j = i / 32 go to the 8 XCDs rotated by j: supers differ in how many of their tiles
+    // exist (partial last column-super, empty tile rows), and a fixed assignment would give some XCDs the full
+    // ones every time.
+    const int j = i / (SM * SN);
+    const int s = j * 8 + ((x + j) & 7), r = i % (SM * SN);
     if (s >= supers) return false;
     ml = r % SM;
     nl = r / SM;
