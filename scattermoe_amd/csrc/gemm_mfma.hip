@@ -836,9 +836,11 @@ struct Raster {
     const int x = pid & 7, i = pid >> 3;
     if (striped) {
       // XCD x owns the tile columns n = x (mod 8) of every tile row; rows slowest, in groups of gm
+      // (the residue class an XCD owns moves on with every group of rows, so that a column count that is not a
+      // multiple of 8 does not leave the same XCDs short every time)
       const int m_lo = i % gm, j = i / gm;
       m = (j / n_supers) * gm + m_lo;
-      n = (j % n_supers) * 8 + x;
+      n = (j % n_supers) * 8 + ((x + j / n_supers) & 7);
       ml = nl = 0;
       return m < m_tiles && n < n_tiles;
     }
