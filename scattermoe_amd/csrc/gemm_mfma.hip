@@ -21,12 +21,12 @@
 //   STRIPE_BELOW average rows per expert under which the 256x256 class uses that order too (Mixtral shape, 1536
 //                tokens: 1.68 -> 1.37 ms for the two forward launches; neutral at 4096, 2 % slower at 8192)
 //   GM_S2S       row super-tiles per raster band of scatter2scatter (4: +3 % on the layer-2 shaped launches)
-//   GM_XTY       the same for groupXtY (unbanded: bands were neutral there)
+//   GM_XTY       the same for groupXtY (4: 1-2 % over unbanded on all three training workloads)
 static constexpr int ROWS32_BELOW = 24, ROWS64_BELOW = 48, ROWS128_BELOW = 112, ROWS256_BELOW = 224;
 static constexpr int GM_RING = 8;
 static constexpr int STRIPE_BELOW = 1024;
 static constexpr int GM_S2S = 4;
-static constexpr int GM_XTY = 1 << 20;
+static constexpr int GM_XTY = 4;
 #include <type_traits>
 
 namespace smoe {
