@@ -23,9 +23,9 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes moved per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (KiB per dispatch, scaled by a copy kernel of known size); None until measured for a workload.
 # c2: average of the two launches of the dominant kernel in a step (layer-1 forward with the gated linear unit
-# in its epilogue 19.25 GB, layer-2 forward 7.48 GB; see profiles/s2s_mfma_c2_l1fwd_counters.md for the commands
+# in its epilogue 17.70 GB, layer-2 forward 7.03 GB; see profiles/s2s_mfma_c2_l1fwd_counters.md for the commands
 # and raw counter values).
-MEASURED_TRAFFIC = {"c2": 13.37e9}
+MEASURED_TRAFFIC = {"c2": 12.36e9}
 
 
 def parse():
