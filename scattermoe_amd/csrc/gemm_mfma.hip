@@ -624,6 +624,11 @@ __device__ __forceinline__ void epilogue_glu_bwd(const f32x16 (&acc)[TL::FM][TL:
 }
 
 // Plain store through LDS: dst[m] is the element offset of output row m of the tile (or -1).
+// Output tiles are written once and not read again by the launch: stored with the non-temporal hint so that they
+// do not displace operand panels in the L2 (c4: -1 % step time, c2: -0.2 %).
+template <typename V>
+__device__ __forceinline__ void stream_store(const V& v, V* p) { __builtin_nontemporal_store(v, p); }
+
 template <typename T, class TL>
 __device__ __forceinline__ void epilogue_staged(const f32x16 (&acc)[TL::FM][TL::FN], T* __restrict__ out,
                                                 const int64_t* dst, int n0, int ncols, const T* __restrict__ bias,
@@ -639,7 +644,7 @@ __device__ __forceinline__ void epilogue_staged(const f32x16 (&acc)[TL::FM][TL::
     const int p = q * TL::NT + threadIdx.x;
     const int row = p / CPR, c = p % CPR, n = n0 + c * 8;
     const int64_t d = dst[row];
-    if (d >= 0 && n < ncols) *(T8*)(out + d + n) = *(const T8*)(lds + staged_addr<TL>(row, c * 8));
+    if (d >= 0 && n < ncols) stream_store(*(const T8*)(lds + staged_addr<TL>(row, c * 8)), (T8*)(out + d + n));
   }
 }
 
@@ -678,10 +683,10 @@ __device__ __forceinline__ void epilogue_glu_fwd_staged(const f32x16 (&acc)[TL::
         h[e] = from_f32<T>(glu_h(a.act, to_f32(gf ? first[e] : second[e]), to_f32(gf ? second[e] : first[e])));
       const int64_t r = row0 + row;
       if (pre != nullptr) {
-        *(T8*)(pre + r * a.sym + n) = first;
-        *(T8*)(pre + r * a.sym + F + n) = second;
+        stream_store(first, (T8*)(pre + r * a.sym + n));
+        stream_store(second, (T8*)(pre + r * a.sym + F + n));
       }
-      *(T8*)(hid + r * a.shm + n) = h;
+      stream_store(h, (T8*)(hid + r * a.shm + n));
     }
   }
 }
@@ -730,8 +735,8 @@ __device__ __forceinline__ void epilogue_glu_bwd_staged(const f32x16 (&acc)[TL::
         o2[e] = gf ? d_lin : d_gat;
       }
       T* dst = dpre + (int64_t)(row0 + row) * a.sym + n;
-      *(T8*)dst = o1;
-      *(T8*)(dst + F) = o2;
+      stream_store(o1, (T8*)dst);
+      stream_store(o2, (T8*)(dst + F));
     }
   }
 }
@@ -762,8 +767,8 @@ __device__ __forceinline__ void epilogue_oss_fwd_staged(const f32x16 (&acc)[TL::
 #pragma unroll
     for (int e = 0; e < 4; ++e) h[e] = from_f32<T>(oss_h(to_f32(v[2 * e]), to_f32(v[2 * e + 1]), a.alpha, a.limit));
     const int64_t r = row0 + row;
-    if (pre != nullptr) *(T8*)(pre + r * a.sym + n) = v;
-    *(T4*)(hid + r * a.shm + n / 2) = h;
+    if (pre != nullptr) stream_store(v, (T8*)(pre + r * a.sym + n));
+    stream_store(h, (T4*)(hid + r * a.shm + n / 2));
   }
 }
 
@@ -812,8 +817,8 @@ __device__ __forceinline__ void epilogue_oss_bwd_staged(const f32x16 (&acc)[TL::
         o2[2 * e + 1] = from_f32<T>(du);
       }
       T* dst = dpre + (int64_t)(row0 + row) * a.sym + 2 * n;
-      *(T8*)dst = o1;
-      *(T8*)(dst + 8) = o2;
+      stream_store(o1, (T8*)dst);
+      stream_store(o2, (T8*)(dst + 8));
     }
   }
 }
