@@ -11,6 +11,20 @@ namespace smoe {
 
 template <typename T> struct Pack { static constexpr int n = 16 / sizeof(T); T v[16 / sizeof(T)]; };
 
+// 16-byte accesses with the non-temporal hint, for data a pass touches exactly once (it should not displace what
+// the neighbouring GEMM launches keep in the caches)
+typedef int nt_i32x4 __attribute__((ext_vector_type(4)));
+template <typename P>
+__device__ __forceinline__ P stream_load16(const void* p) {
+  static_assert(sizeof(P) == 16, "16-byte packs only");
+  return __builtin_bit_cast(P, __builtin_nontemporal_load((const nt_i32x4*)p));
+}
+template <typename P>
+__device__ __forceinline__ void stream_store16(void* p, const P& x) {
+  static_assert(sizeof(P) == 16, "16-byte packs only");
+  __builtin_nontemporal_store(__builtin_bit_cast(nt_i32x4, x), (nt_i32x4*)p);
+}
+
 // ---- combine -------------------------------------------------------------------------------------------
 template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void combine_kernel(const T* __restrict__ Y, int64_t sy, const T* __restrict__ G,
@@ -26,7 +40,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const T* __restrict__ Y, i
       for (int q = 0; q < P::n; ++q) acc[q] = 0.0f;
       for (int j = 0; j < k; ++j) {
         const float g = to_f32(G[t * sgt + j * sgk]);
-        const P x = *(const P*)(y0 + j * sy + (int64_t)c * P::n);
+        const P x = stream_load16<P>(y0 + j * sy + (int64_t)c * P::n);
 #pragma unroll
         for (int q = 0; q < P::n; ++q) acc[q] = fmaf(g, to_f32(x.v[q]), acc[q]);
       }
@@ -59,7 +73,7 @@ __global__ __launch_bounds__(256) void gate_grad_kernel(const T* __restrict__ Y,
     if (VEC) {
       typedef Pack<T> P;
       for (int c = threadIdx.x; c < N / P::n; c += 256) {
-        const P a = *(const P*)(y + (int64_t)c * P::n);
+        const P a = stream_load16<P>(y + (int64_t)c * P::n);
         const P b = *(const P*)(d + (int64_t)c * P::n);
 #pragma unroll
         for (int q = 0; q < P::n; ++q) acc = fmaf(to_f32(a.v[q]), to_f32(b.v[q]), acc);
@@ -90,12 +104,12 @@ __global__ __launch_bounds__(256) void glu_fwd_kernel(const T* __restrict__ pre,
     const int64_t r = i / per_row, c = (i % per_row) * W;
     if (VEC) {
       typedef Pack<T> P;
-      const P lin = *(const P*)(pre + r * sp + (gf ? f : 0) + c);
-      const P gat = *(const P*)(pre + r * sp + (gf ? 0 : f) + c);
+      const P lin = stream_load16<P>(pre + r * sp + (gf ? f : 0) + c);
+      const P gat = stream_load16<P>(pre + r * sp + (gf ? 0 : f) + c);
       P o;
 #pragma unroll
       for (int q = 0; q < P::n; ++q) o.v[q] = from_f32<T>(glu_h(act, to_f32(gat.v[q]), to_f32(lin.v[q])));
-      *(P*)(h + r * sh + c) = o;
+      stream_store16(h + r * sh + c, o);
     } else {
       h[r * sh + c] = from_f32<T>(glu_h(act, to_f32(pre[r * sp + (gf ? 0 : f) + c]), to_f32(pre[r * sp + (gf ? f : 0) + c])));
     }
@@ -114,9 +128,9 @@ __global__ __launch_bounds__(256) void glu_bwd_kernel(const T* __restrict__ pre,
     const int64_t r = i / per_row, c = (i % per_row) * W;
     if (VEC) {
       typedef Pack<T> P;
-      const P lin = *(const P*)(pre + r * sp + (gf ? f : 0) + c);
-      const P gat = *(const P*)(pre + r * sp + (gf ? 0 : f) + c);
-      const P d = *(const P*)(dh + r * sdh + c);
+      const P lin = stream_load16<P>(pre + r * sp + (gf ? f : 0) + c);
+      const P gat = stream_load16<P>(pre + r * sp + (gf ? 0 : f) + c);
+      const P d = stream_load16<P>(dh + r * sdh + c);
       P ol, og;
 #pragma unroll
       for (int q = 0; q < P::n; ++q) {
@@ -124,8 +138,8 @@ __global__ __launch_bounds__(256) void glu_bwd_kernel(const T* __restrict__ pre,
         ol.v[q] = from_f32<T>(glu_dlin(act, dv, g));
         og.v[q] = from_f32<T>(glu_dgat(act, dv, g, to_f32(lin.v[q])));
       }
-      *(P*)(dpre + r * sdp + (gf ? f : 0) + c) = ol;
-      *(P*)(dpre + r * sdp + (gf ? 0 : f) + c) = og;
+      stream_store16(dpre + r * sdp + (gf ? f : 0) + c, ol);
+      stream_store16(dpre + r * sdp + (gf ? 0 : f) + c, og);
     } else {
       const float g = to_f32(pre[r * sp + (gf ? 0 : f) + c]), dv = to_f32(dh[r * sdh + c]);
       dpre[r * sdp + (gf ? f : 0) + c] = from_f32<T>(glu_dlin(act, dv, g));
@@ -148,7 +162,7 @@ __global__ __launch_bounds__(256) void oss_glu_fwd_kernel(const T* __restrict__ 
     const int64_t r = i / per_row, c = (i % per_row) * W;
     if (VEC) {
       struct Half { T v[W]; };
-      const Pack<T> p = *(const Pack<T>*)(pre + r * sp + 2 * c);
+      const Pack<T> p = stream_load16<Pack<T>>(pre + r * sp + 2 * c);
       Half o;
 #pragma unroll
       for (int q = 0; q < W; ++q) o.v[q] = from_f32<T>(oss_h(to_f32(p.v[2 * q]), to_f32(p.v[2 * q + 1]), alpha, limit));
@@ -169,7 +183,7 @@ __global__ __launch_bounds__(256) void oss_glu_bwd_kernel(const T* __restrict__ 
     const int64_t r = i / per_row, c = (i % per_row) * W;
     if (VEC) {
       struct Half { T v[W]; };
-      const Pack<T> p = *(const Pack<T>*)(pre + r * sp + 2 * c);
+      const Pack<T> p = stream_load16<Pack<T>>(pre + r * sp + 2 * c);
       const Half d = *(const Half*)(dh + r * sdh + c);
       Pack<T> o;
 #pragma unroll
@@ -179,7 +193,7 @@ __global__ __launch_bounds__(256) void oss_glu_bwd_kernel(const T* __restrict__ 
         o.v[2 * q] = from_f32<T>(dg);
         o.v[2 * q + 1] = from_f32<T>(du);
       }
-      *(Pack<T>*)(dpre + r * sdp + 2 * c) = o;
+      stream_store16(dpre + r * sdp + 2 * c, o);
     } else {
       float dg, du;
       oss_grad(to_f32(pre[r * sp + 2 * c]), to_f32(pre[r * sp + 2 * c + 1]), to_f32(dh[r * sdh + c]), alpha, limit, dg, du);

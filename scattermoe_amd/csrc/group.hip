@@ -28,6 +28,7 @@ __global__ __launch_bounds__(kGroupThreads) void group_kernel(GroupArgs a) {
     T* __restrict__ d = Y + n * a.sym;
     if (VEC) {
       typedef Vec16<T> V;
+      typedef int VV __attribute__((ext_vector_type(4)));
       const int nv = a.K / V::n;
       for (int j = lane; j < nv; j += 64) {
         V x = *(const V*)(s + (int64_t)j * V::n);
@@ -35,7 +36,7 @@ __global__ __launch_bounds__(kGroupThreads) void group_kernel(GroupArgs a) {
 #pragma unroll
           for (int q = 0; q < V::n; ++q) x.v[q] = from_f32<T>(to_f32(x.v[q]) * c);
         }
-        *(V*)(d + (int64_t)j * V::n) = x;
+        __builtin_nontemporal_store(*(const VV*)&x, (VV*)(d + (int64_t)j * V::n));
       }
     } else {
       for (int j = lane; j < a.K; j += 64) {
