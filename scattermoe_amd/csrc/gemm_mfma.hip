@@ -88,11 +88,20 @@ typedef __attribute__((address_space(1))) const void glb_void_t;
 // matters: the same load with a full 64-bit address in each lane costs the issuing wave so much issue time
 // that the matrix pipe starves (measured: +50% run time for 8 such loads per 32 MFMAs, against no
 // measurable cost for the scalar-base form).
+// STREAM: the non-temporal hint, for an operand the launch reads exactly once (the weights of the memory-bound
+// classes), so that it does not displace the rows that are read again and again.
+template <bool STREAM = false>
 __device__ __forceinline__ void load_to_lds16(const char* base_uniform, unsigned off, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-               :
-               : "s"(lds_addr), "v"(off), "s"(base_uniform)
-               : "memory", "m0");
+  if constexpr (STREAM)
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
+                 :
+                 : "s"(lds_addr), "v"(off), "s"(base_uniform)
+                 : "memory", "m0");
+  else
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_addr), "v"(off), "s"(base_uniform)
+                 : "memory", "m0");
 }
 __device__ __forceinline__ const char* make_uniform(const char* p) {
   const uint64_t v = (uint64_t)p;
@@ -111,7 +120,7 @@ __device__ __forceinline__ const char* make_uniform(const char* p) {
 // phase (16 consecutive rows, one chunk) hit 16 different 16-byte bank groups.
 __device__ __forceinline__ int direct_swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
-template <int EXT, int NT>
+template <int EXT, int NT, bool STREAM = false>
 struct DirectOp {
   static constexpr int PIECES = EXT * 8;
   static constexpr int R = PIECES / NT;
@@ -138,7 +147,7 @@ struct DirectOp {
     }
   }
   __device__ __forceinline__ void issue_one(unsigned tile, int k0, int j) const {
-    load_to_lds16(base + (int64_t)k0 * 2, off[j], tile + wave_uniform_id() * 1024 + rnd(j) * NT * 16);
+    load_to_lds16<STREAM>(base + (int64_t)k0 * 2, off[j], tile + wave_uniform_id() * 1024 + rnd(j) * NT * 16);
   }
   __device__ __forceinline__ void issue(unsigned tile, int k0) const {
 #pragma unroll
@@ -150,7 +159,7 @@ struct DirectOp {
     const int p = rnd(j) * NT + threadIdx.x;
     const int c = (p & 7) ^ direct_swz(p >> 3);
     const bool ok = k0 + c * 8 < kend;
-    load_to_lds16(base, ok ? off[j] + (unsigned)k0 * 2 : off[j] - (c << 4),
+    load_to_lds16<STREAM>(base, ok ? off[j] + (unsigned)k0 * 2 : off[j] - (c << 4),
                   tile + wave_uniform_id() * 1024 + rnd(j) * NT * 16);
   }
   __device__ __forceinline__ void issue_tail(unsigned tile, int k0, int kend) const {
@@ -178,7 +187,7 @@ struct DirectOp {
 // Row kr of the tile is EXT*2 bytes = G granules of 64 B (32 columns).  A ds_read_b64_tr_b16 phase touches
 // one granule column in 4 consecutive rows; storing granule g of row kr at position g ^ (kr & 3) spreads
 // those 4 accesses over all 64 banks.
-template <int EXT, int NT>
+template <int EXT, int NT, bool STREAM = false>
 struct TransOp {
   static constexpr int CPR = EXT / 8;                  // 16-byte pieces per contraction row
   static constexpr int PIECES = 64 * CPR;
@@ -212,7 +221,7 @@ struct TransOp {
     }
   }
   __device__ __forceinline__ void issue_one(unsigned tile, int k0, int j) const {
-    load_to_lds16(base + (int64_t)k0 * ld, off[j], tile + wave_uniform_id() * 1024 + rnd(j) * NT * 16);
+    load_to_lds16<STREAM>(base + (int64_t)k0 * ld, off[j], tile + wave_uniform_id() * 1024 + rnd(j) * NT * 16);
   }
   __device__ __forceinline__ void issue(unsigned tile, int k0) const {
 #pragma unroll
@@ -223,7 +232,7 @@ struct TransOp {
   __device__ __forceinline__ void issue_tail_one(unsigned tile, int k0, int kend, int j) const {
     const int kr = (rnd(j) * NT + (int)threadIdx.x) / CPR;
     const bool ok = k0 + kr < kend;
-    load_to_lds16(base + (int64_t)k0 * ld, ok ? off[j] : off[j] - (unsigned)(kr * ld),
+    load_to_lds16<STREAM>(base + (int64_t)k0 * ld, ok ? off[j] : off[j] - (unsigned)(kr * ld),
                   tile + wave_uniform_id() * 1024 + rnd(j) * NT * 16);
   }
   __device__ __forceinline__ void issue_tail(unsigned tile, int k0, int kend) const {
@@ -908,7 +917,8 @@ static Raster make_striped(int64_t m_tiles, int n_tiles, int gm) {
 template <typename T, class TL, bool B_TR>
 __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast) {
   typedef DirectOp<TL::BM, TL::NT> AOp;
-  typedef typename std::conditional<B_TR, TransOp<TL::BN, TL::NT>, DirectOp<TL::BN, TL::NT>>::type BOp;
+  constexpr bool W_ONCE = TL::NS > 2 && TL::BM <= 64;      // few rows per expert: every weight element is read once
+  typedef typename std::conditional<B_TR, TransOp<TL::BN, TL::NT, W_ONCE>, DirectOp<TL::BN, TL::NT, W_ONCE>>::type BOp;
   constexpr int STAGE = AOp::LDS_BYTES + BOp::LDS_BYTES;
   __shared__ __attribute__((aligned(16))) char lds[TL::NS * STAGE];
   __shared__ int64_t sDst[TL::BM];

@@ -71,7 +71,7 @@ __device__ __forceinline__ void rowdot_pass(const char* Xb, const int64_t (&xoff
   for (int k = (wave * 64 + lane) * 8; k < K; k += NW * RD_PIECE) {
     u32x4 w[C], x[R];
 #pragma unroll
-    for (int c = 0; c < C; ++c) w[c] = *(const u32x4*)(wp[c] + (int64_t)k * 2);
+    for (int c = 0; c < C; ++c) w[c] = __builtin_nontemporal_load((const u32x4*)(wp[c] + (int64_t)k * 2));   // read once
 #pragma unroll
     for (int r = 0; r < R; ++r) x[r] = *(const u32x4*)(Xb + xoff[r] + (int64_t)k * 2);
 #pragma unroll
