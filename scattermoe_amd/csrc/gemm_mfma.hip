@@ -22,7 +22,7 @@
 //                tokens: 1.68 -> 1.37 ms for the two forward launches; neutral at 4096, 2 % slower at 8192)
 //   GM_S2S       row super-tiles per raster band of scatter2scatter (4: +3 % on the layer-2 shaped launches)
 //   GM_XTY       the same for groupXtY (4: 1-2 % over unbanded on all three training workloads)
-static constexpr int ROWS32_BELOW = 24, ROWS64_BELOW = 48, ROWS128_BELOW = 112, ROWS256_BELOW = 224;
+static constexpr int ROWS32_BELOW = 24, ROWS64_BELOW = 52, ROWS128_BELOW = 112, ROWS256_BELOW = 224;
 static constexpr int GM_RING = 8;
 static constexpr int STRIPE_BELOW = 1024;
 static constexpr int GM_S2S = 4;

@@ -19,7 +19,7 @@ SHAPES = [
     (2048, 4, 2, 256, 384),      # 1024 rows/expert: 256-row tiles, exact multiples
     (1100, 8, 2, 200, 264),      # 275 rows/expert: ragged rows, d % 64 != 0, F % 128 != 0
     (520, 8, 2, 320, 1000),      # 130 rows/expert: ring-buffered 256x128 tiles
-    (130, 8, 3, 448, 72),        # ~49 rows/expert: ring-buffered 128x128 tiles, F < one tile
+    (160, 8, 3, 448, 72),        # 60 rows/expert: ring-buffered 128x128 tiles, F < one tile
     (130, 8, 2, 320, 200),       # ~32 rows/expert: 64-row ring tiles
     (40, 8, 2, 192, 136),        # 10 rows/expert: no fused forward kernel (falls back), fused backward
 ]

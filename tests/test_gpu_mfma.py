@@ -36,7 +36,7 @@ SHAPES = [
     (4096, 8, 2, 512, 768),      # 1024 rows/expert: 256x256 tiles, exact multiples
     (1100, 8, 2, 200, 264),      # 275 rows/expert: ragged row tails, K % 64 != 0, N % 256 != 0
     (520, 8, 2, 320, 1000),      # 130 rows/expert: ring-buffered 256x128 tiles
-    (130, 8, 3, 448, 72),        # ~49 rows/expert: ring-buffered 128x128 tiles, N < one tile
+    (160, 8, 3, 448, 72),        # 60 rows/expert: ring-buffered 128x128 tiles, N < one tile
     (300, 8, 2, 200, 328),       # 75 rows/expert: 128x128 ring tiles with contraction and column tails
     (130, 8, 2, 448, 200),       # ~32 rows/expert: 64-row ring tiles
     (3, 8, 2, 64, 256),          # decode-like: a handful of rows (ring-buffered 32-row tiles)
