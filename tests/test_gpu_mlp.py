@@ -148,3 +148,22 @@ def test_module_random_shapes(T, E, k, d, f, kind, bias, dtype, skew):
     rtol, atol = (1e-4, 1e-5) if dtype == torch.float32 else (2e-2, 1e-2)
     for n, a, b in _run_pair(m, x, p, experts, dy, dtype):
         _rel_check(n, a, b, rtol, atol)
+
+
+@pytest.mark.parametrize("dtype,T", [(torch.float32, 300), (torch.bfloat16, 300), (torch.bfloat16, 3)])
+def test_mixture_of_lora_shape(dtype, T):
+    """The module of the reference's example (examples/molora.py:5-17): 16 rank-128 adapters over d = 1024 with
+    an identity between the two layers, forward and every gradient."""
+    d, rank, E, k = 1024, 128, 16, 2
+    g = torch.Generator().manual_seed(T)
+    p, experts = torch.topk(torch.softmax(torch.randn(T, E, generator=g), -1), k)
+    x = torch.randn(T, d, generator=g)
+    dy = torch.randn(T, d, generator=g)
+    torch.manual_seed(5)
+    m = MLP(d, rank, E, k, activation=nn.Identity())
+    with torch.no_grad():
+        for prm in m.parameters():
+            prm.normal_(0, 0.05)
+    rtol, atol = (1e-4, 1e-5) if dtype == torch.float32 else (2e-2, 1e-2)
+    for n, a, b in _run_pair(m, x, p, experts, dy, dtype, per_token=(T < 8)):
+        _rel_check(n, a, b, rtol, atol)

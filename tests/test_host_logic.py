@@ -122,6 +122,16 @@ def test_api_surface_and_errors(cpu_backend):
         ops.scatter2scatter(torch.randn(2, 4), torch.randn(2, 4, 4), eid, idx, 2, out=torch.empty(4, 5))
 
 
+def test_mixture_of_lora_module_prints_like_the_reference():
+    """The module of the reference's example (examples/molora.py:5-24) and the text it prints there."""
+    import scattermoe_amd as sm
+    m = sm.mlp.MLP(input_size=1024, hidden_size=128, num_experts=16, top_k=2, activation=nn.Identity())
+    assert repr(m) == ("MLP(\n  k=2\n"
+                       "  (experts): ParallelExperts(num_experts=16, input_size=1024, output_size=128)\n"
+                       "  (output_experts): ParallelExperts(num_experts=16, input_size=128, output_size=1024)\n"
+                       "  (activation): Identity()\n)")
+
+
 def test_product_path_refuses_cpu_tensors():
     """Without the test double the launch layer is the HIP library and must not silently run on CPU."""
     import scattermoe_amd as sm
