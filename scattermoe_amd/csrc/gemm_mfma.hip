@@ -28,6 +28,7 @@ static constexpr int STRIPE_BELOW = 1024;
 static constexpr int GM_S2S = 4;
 static constexpr int GM_XTY = 4;
 #include <type_traits>
+#include <math.h>
 
 namespace smoe {
 
@@ -1031,6 +1032,27 @@ static int launch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
   return launch_status("s2s_mfma_kernel");
 }
 
+// Launches of only a few rounds of 256 x 256 tiles (one tile per CU and round) lose up to a whole round to the
+// partly filled last one; tiles of half the width take HALF_WIDTH_COST of the time and round off finer.  The
+// number of tile rows is only known on the device; the host prices both classes with its expectation for rows
+// spread evenly over the experts (binomial spread around the mean).  A wrong guess costs speed only.  Mixtral
+// expert shapes, layer 1 + layer 2 forward: 896 tokens 912 -> 833 us, 1984..2112 tokens -3 %, nothing lost
+// anywhere between 800 and 3136 tokens.
+static constexpr int NUM_CU = 256;
+static constexpr double HALF_WIDTH_COST = 0.58;
+static bool half_width_wins(const S2SArgs& a) {
+  const int cols = a.glu == 1 ? 128 : 256;               // output columns of a 256-wide tile
+  const int64_t n_full = (a.N + cols - 1) / cols, n_half = (a.N + cols / 2 - 1) / (cols / 2);
+  if (max_tiles(a.L, a.E, 256) * n_full > 4 * NUM_CU) return false;
+  const double avg = (double)a.L / a.E, sd = sqrt(avg * (1.0 - 1.0 / a.E)) + 1e-9;
+  double per_expert = 1.0;                               // expected ceil(rows / 256)
+  for (int j = 1; j * 256.0 < avg + 6 * sd; ++j) per_expert += 0.5 * erfc((j * 256.0 - avg) / (sd * 1.41421356));
+  const double m = nearbyint(per_expert * a.E);
+  if (m * n_full < 96) return false;                     // far below one round: nothing to win, keep the default
+  const double full = ceil(m * n_full / NUM_CU), half = ceil(m * n_half / NUM_CU) * HALF_WIDTH_COST;
+  return half < 0.95 * full;
+}
+
 template <typename T>
 static int dispatch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
   // the gpt-oss epilogues exist only in their LDS-staged form (16-byte pieces)
@@ -1040,7 +1062,7 @@ static int dispatch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
   if (a.glu == 4 && !((((uintptr_t)a.aux | (uintptr_t)a.Y) & 15) == 0 && ((a.saux | a.sym | a.N) & 7) == 0))
     return SMOE_ERR_UNSUPPORTED;
   const int64_t avg = a.L / a.E;
-  if (avg >= ROWS256_BELOW) return launch_s2s<T, Tile<256, 256, 2, 4>>(a, b_tr, st);
+  if (avg >= ROWS256_BELOW && !half_width_wins(a)) return launch_s2s<T, Tile<256, 256, 2, 4>>(a, b_tr, st);
   // Below that the launch is a stream over the weights: ring-buffered classes, tile height by rows per expert
   if (avg >= ROWS128_BELOW) return launch_s2s<T, Tile<256, 128, 4, 2, 3>>(a, b_tr, st);
   if (avg >= ROWS32_BELOW && avg < ROWS64_BELOW) return launch_s2s<T, Tile<64, 128, 2, 2, 5>>(a, b_tr, st);

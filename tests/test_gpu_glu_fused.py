@@ -22,6 +22,7 @@ SHAPES = [
     (160, 8, 3, 448, 72),        # 60 rows/expert: ring-buffered 128x128 tiles, F < one tile
     (130, 8, 2, 320, 200),       # ~32 rows/expert: 64-row ring tiles
     (40, 8, 2, 192, 136),        # 10 rows/expert: no fused forward kernel (falls back), fused backward
+    (960, 8, 2, 64, 2048),       # 240 rows/expert, about half a round of 256-row tiles: half-width tiles chosen
 ]
 
 

@@ -44,6 +44,7 @@ SHAPES = [
     (9, 4, 2, 1096, 136),        # 32-row tiles, contraction longer than the ring (17 full slices + tail)
     (40, 8, 2, 200, 1288),       # enough 128-wide tiles to pick the 64-wide ring class for K-contiguous weights
     (2048, 32, 4, 192, 328),     # E = 32 with skew: tiny and empty experts
+    (960, 8, 2, 64, 4096),       # 240 rows/expert, about half a round of 256x256 tiles: half-width tiles chosen
 ]
 
 
