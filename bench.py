@@ -22,10 +22,10 @@ PEAK_HBM_GBS = 8000.0
 
 # HBM bytes moved per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (KiB per dispatch, scaled by a copy kernel of known size); None until measured for a workload.
-# c2: average of the two launches of the dominant kernel in a step (layer-1 forward with the gated linear unit
-# in its epilogue 17.70 GB, layer-2 forward 7.03 GB; see profiles/s2s_mfma_c2_l1fwd_counters.md for the commands
+# c2: average over the two products of the dominant kernel in a step (layer-1 forward with the gated linear unit
+# in its epilogue 21.33 GB, layer-2 forward 7.49 GB; see profiles/s2s_mfma_c2_l1fwd_counters.md for the commands
 # and raw counter values).
-MEASURED_TRAFFIC = {"c2": 12.36e9}
+MEASURED_TRAFFIC = {"c2": 14.41e9}
 
 
 def parse():
@@ -273,7 +273,8 @@ def main():
     achieved = k_fl / (k_ms * 1e-3) / 1e12
     roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": MEASURED_TRAFFIC.get(cfg.name),
-                "kernel": "s2s_mfma_kernel (scatter2scatter, K-contiguous weights)",
+                "kernel": "s2s_mfma_kernel (scatter2scatter products with K-contiguous weights; a product of a few "
+                          "rounds of tiles plus a remainder runs as two launches and is timed as one)",
                 "launches_per_step": len(sel) // args.steps, "avg_launch_ms": round(k_ms, 4),
                 "avg_flop_per_launch": k_fl,
                 "all_s2s_launches_avg_tflops": round(sum(fl for _, fl in allk) / sum(t for t, _ in allk) / 1e9, 1)}

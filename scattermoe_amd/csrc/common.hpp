@@ -149,6 +149,9 @@ struct S2SArgs {
   const void* aux = nullptr; int64_t saux = 0;
   void* H = nullptr; int64_t shm = 0;
   float alpha = 0.0f, limit = 0.0f;
+  // Part of a product split by tile rows (MFMA path only): the launch covers the tile rows
+  // [m_begin, m_begin + m_count) of its tile height.
+  int m_begin = 0, m_count = 0x7fffffff;
 };
 
 struct XtYArgs {

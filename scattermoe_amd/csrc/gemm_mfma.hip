@@ -28,6 +28,7 @@ static constexpr int STRIPE_BELOW = 1024;
 static constexpr int GM_S2S = 4;
 static constexpr int GM_XTY = 4;
 #include <type_traits>
+#include <algorithm>
 #include <math.h>
 
 namespace smoe {
@@ -928,7 +929,7 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
   int m_tile, n_tile, m_loc, n_loc;
   if (!rast.map(blockIdx.x, m_tile, n_tile, m_loc, n_loc)) return;
   int e, row0, rows;
-  if (!find_tile<TL::BM>(a.off, a.E, m_tile, e, row0, rows)) return;
+  if (m_tile >= a.m_count || !find_tile<TL::BM>(a.off, a.E, a.m_begin + m_tile, e, row0, rows)) return;
   // first output column of the tile; the fused forward GLU tile holds BN/2 columns of each half
   const int n0 = a.glu == 1 ? n_tile * (TL::BN / 2) : n_tile * TL::BN;
 
@@ -1015,7 +1016,7 @@ template <typename T, class TL>
 static int launch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
   const int bn = a.glu == 1 ? TL::BN / 2 : TL::BN;     // output columns per tile
   const int n_tiles = (a.N + bn - 1) / bn;
-  const int64_t m_tiles = max_tiles(a.L, a.E, TL::BM);
+  const int64_t m_tiles = std::min<int64_t>(max_tiles(a.L, a.E, TL::BM) - a.m_begin, a.m_count);
   // With only a few tile rows per expert no weight panel is shared by the tile rows of a super tile; the striped
   // order at least keeps the tile rows of one expert together on one XCD.
   const bool striped = TL::NS > 2 || a.L / a.E < STRIPE_BELOW;
@@ -1040,17 +1041,42 @@ static int launch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
 // anywhere between 800 and 3136 tokens.
 static constexpr int NUM_CU = 256;
 static constexpr double HALF_WIDTH_COST = 0.58;
+// expected number of 256-row tiles, rounded
+static double expected_row_tiles(int64_t L, int E) {
+  const double avg = (double)L / E, sd = sqrt(avg * (1.0 - 1.0 / E)) + 1e-9;
+  double per_expert = 1.0;                               // expected ceil(rows / 256)
+  for (int j = 1; j * 256.0 < avg + 6 * sd; ++j) per_expert += 0.5 * erfc((j * 256.0 - avg) / (sd * 1.41421356));
+  return nearbyint(per_expert * E);
+}
 static bool half_width_wins(const S2SArgs& a) {
   const int cols = a.glu == 1 ? 128 : 256;               // output columns of a 256-wide tile
   const int64_t n_full = (a.N + cols - 1) / cols, n_half = (a.N + cols / 2 - 1) / (cols / 2);
   if (max_tiles(a.L, a.E, 256) * n_full > 4 * NUM_CU) return false;
-  const double avg = (double)a.L / a.E, sd = sqrt(avg * (1.0 - 1.0 / a.E)) + 1e-9;
-  double per_expert = 1.0;                               // expected ceil(rows / 256)
-  for (int j = 1; j * 256.0 < avg + 6 * sd; ++j) per_expert += 0.5 * erfc((j * 256.0 - avg) / (sd * 1.41421356));
-  const double m = nearbyint(per_expert * a.E);
+  const double m = expected_row_tiles(a.L, a.E);
   if (m * n_full < 96) return false;                     // far below one round: nothing to win, keep the default
   const double full = ceil(m * n_full / NUM_CU), half = ceil(m * n_half / NUM_CU) * HALF_WIDTH_COST;
   return half < 0.95 * full;
+}
+
+// A launch of a few whole rounds plus a remainder of up to half a round pays a whole round for the remainder.
+// Such a product is cut by tile rows: the whole rounds stay with the 256 x 256 class, the remaining tile rows go
+// to a second launch of 256 x 128 tiles (twice the workgroups, 0.58 of the time).  Returns the number of tile
+// rows of the first launch, 0 when the product is not split.  Plain products only (no fused unit behind them).
+// Mixtral shape, 16384 tokens (8.25 rounds in the launches with 4096 output columns): layer-2 forward
+// 3.47 -> 3.34 ms, layer-1 input gradient 7.03 -> 6.68 ms; 128 x 128 tiles for the remainder were slower
+// (four times the workgroups at 0.75 of the time).
+static int tail_split(const S2SArgs& a) {
+  if (a.glu != 0 || a.m_begin != 0) return 0;
+  const int64_t n_full = (a.N + 255) / 256;
+  const int64_t upper = max_tiles(a.L, a.E, 256);
+  if (upper * n_full > 26 * NUM_CU) return 0;
+  const double m = expected_row_tiles(a.L, a.E);
+  const int64_t whole = (int64_t)(m * n_full) / NUM_CU;           // whole rounds
+  if (whole < 2) return 0;
+  const int64_t m_first = whole * NUM_CU / n_full;                // tile rows that fit the whole rounds
+  const int64_t rest = ((int64_t)m - m_first) * n_full;           // expected 256 x 256 tiles of the remainder
+  if (m_first <= 0 || rest <= 0 || upper <= m_first || rest > NUM_CU / 2 + 8) return 0;
+  return (int)m_first;
 }
 
 template <typename T>
@@ -1062,6 +1088,13 @@ static int dispatch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
   if (a.glu == 4 && !((((uintptr_t)a.aux | (uintptr_t)a.Y) & 15) == 0 && ((a.saux | a.sym | a.N) & 7) == 0))
     return SMOE_ERR_UNSUPPORTED;
   const int64_t avg = a.L / a.E;
+  if (const int m_first = avg >= ROWS256_BELOW ? tail_split(a) : 0) {
+    S2SArgs first = a, rest = a;
+    first.m_count = m_first;
+    rest.m_begin = m_first;
+    if (const int rc = launch_s2s<T, Tile<256, 256, 2, 4>>(first, b_tr, st)) return rc;
+    return launch_s2s<T, Tile<256, 128, 4, 2, 3>>(rest, b_tr, st);
+  }
   if (avg >= ROWS256_BELOW && !half_width_wins(a)) return launch_s2s<T, Tile<256, 256, 2, 4>>(a, b_tr, st);
   // Below that the launch is a stream over the weights: ring-buffered classes, tile height by rows per expert
   if (avg >= ROWS128_BELOW) return launch_s2s<T, Tile<256, 128, 4, 2, 3>>(a, b_tr, st);

@@ -89,6 +89,36 @@ def test_s2s_modes(x_grouped, y_grouped, w_layout):
     assert torch.equal(got, again)
 
 
+@pytest.mark.parametrize("w_layout", ["k_contig", "n_contig"])
+@pytest.mark.parametrize("x_grouped,y_grouped", list(itertools.product([False, True], repeat=2)))
+@pytest.mark.parametrize("T,skew", [(4000, 0.0), (4200, 0.0), (4000, 1.0)])
+def test_s2s_launch_split_by_tile_rows(T, skew, x_grouped, y_grouped, w_layout):
+    """Two whole rounds of 256 x 256 tiles plus a remainder of up to half a round (T = 4000: 32 expected remaining
+    tiles, T = 4200: 96): the product is cut by tile rows and the remainder goes to a launch of 256 x 128 tiles;
+    with skewed routing the host's expectation of the tile rows is off.  Every output row must be written exactly
+    once, and each element must be the same bits as in the launches over the two column halves, which are not
+    split."""
+    E, k, K, N = 8, 2, 64, 4096
+    experts, (eid, idx, off) = _routing(T, E, k, seed=T, skew=skew)
+    g = torch.Generator().manual_seed(T + 1)
+    fan = 1 if x_grouped else k
+    X = torch.randn(T * k // fan, K, generator=g).bfloat16()
+    Wp = (torch.randn(E, N, K, generator=g) * 0.1).bfloat16()
+    b = torch.randn(E, N, generator=g).bfloat16()
+    Wd = Wp.to(DEV).permute(0, 2, 1)
+    if w_layout == "n_contig":
+        Wd = Wd.contiguous()
+    args = (eid.to(DEV), idx.to(DEV), fan)
+    kw = dict(x_grouped=x_grouped, y_grouped=y_grouped, expert_offsets=off.to(DEV))
+    out = torch.full((T * k, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    got = ops.scatter2scatter(X.to(DEV), Wd, *args, b=b.to(DEV), out=out, **kw)
+    want = oracle.scatter2scatter_ref(X.float(), Wp.permute(0, 2, 1).float(), eid, idx, fan, b.float(), x_grouped, y_grouped)
+    _close(got, want, scale=0.1 * K ** 0.5)
+    halves = [ops.scatter2scatter(X.to(DEV), Wd[:, :, c:c + N // 2], *args, b=b.to(DEV)[:, c:c + N // 2], **kw)
+              for c in (0, N // 2)]
+    assert torch.equal(got, torch.cat(halves, 1))
+
+
 def test_s2s_strided_rows():
     """X and Y that are column slices of wider buffers (row stride != width)."""
     T, E, k, K, N = 600, 8, 2, 128, 256
