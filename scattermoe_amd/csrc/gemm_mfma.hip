@@ -1092,6 +1092,7 @@ static int dispatch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
     S2SArgs first = a, rest = a;
     first.m_count = m_first;
     rest.m_begin = m_first;
+    // both classes have 256-row tiles, hence the same numbering of the tile rows
     if (const int rc = launch_s2s<T, Tile<256, 256, 2, 4>>(first, b_tr, st)) return rc;
     return launch_s2s<T, Tile<256, 128, 4, 2, 3>>(rest, b_tr, st);
   }
