@@ -1044,8 +1044,10 @@ static constexpr double HALF_WIDTH_COST = 0.58;
 // expected number of 256-row tiles, rounded
 static double expected_row_tiles(int64_t L, int E) {
   const double avg = (double)L / E, sd = sqrt(avg * (1.0 - 1.0 / E)) + 1e-9;
-  double per_expert = 1.0;                               // expected ceil(rows / 256)
-  for (int j = 1; j * 256.0 < avg + 6 * sd; ++j) per_expert += 0.5 * erfc((j * 256.0 - avg) / (sd * 1.41421356));
+  // expected ceil(rows / 256) = 1 + sum_j P(rows > 256 j); the terms more than 6 sd below the mean are 1
+  const int j_lo = std::max(1, (int)((avg - 6 * sd) / 256.0));
+  double per_expert = j_lo;
+  for (int j = j_lo; j * 256.0 < avg + 6 * sd; ++j) per_expert += 0.5 * erfc((j * 256.0 - avg) / (sd * 1.41421356));
   return nearbyint(per_expert * E);
 }
 static bool half_width_wins(const S2SArgs& a) {
