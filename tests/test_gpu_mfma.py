@@ -7,6 +7,7 @@ import pytest
 import torch
 
 import oracle
+import scattermoe_amd as sm
 from scattermoe_amd.kernels import ops
 
 pytestmark = pytest.mark.gpu
@@ -117,6 +118,39 @@ def test_s2s_launch_split_by_tile_rows(T, skew, x_grouped, y_grouped, w_layout):
     halves = [ops.scatter2scatter(X.to(DEV), Wd[:, :, c:c + N // 2], *args, b=b.to(DEV)[:, c:c + N // 2], **kw)
               for c in (0, N // 2)]
     assert torch.equal(got, torch.cat(halves, 1))
+
+
+def test_split_product_replays_from_a_graph():
+    """A product that runs as two launches (see the test above), routing included, captured into a HIP graph and
+    replayed on fresh inputs, with eager work between the replays: every replay equals the eager result."""
+    T, E, k, K, N = 4000, 8, 2, 64, 4096
+    g = torch.Generator().manual_seed(3)
+    W = (torch.randn(E, N, K, generator=g) * 0.1).bfloat16().to(DEV).permute(0, 2, 1)
+    X = torch.randn(T, K, generator=g).bfloat16().to(DEV)
+    experts = torch.topk(torch.randn(T, E, generator=g), k).indices.to(DEV)
+
+    def step():
+        eid, idx, off = sm.flatten_sort_count(experts, E)
+        return ops.scatter2scatter(X, W, eid, idx, k, expert_offsets=off)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y_static = step()
+    for r in range(3):
+        X.copy_(torch.randn(T, K, generator=g).bfloat16())
+        experts.copy_(torch.topk(torch.randn(T, E, generator=g), k).indices)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = y_static.clone()
+        want = step()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), "replay %d differs from the eager result" % r
 
 
 def test_s2s_strided_rows():
