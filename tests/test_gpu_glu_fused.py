@@ -23,6 +23,7 @@ SHAPES = [
     (130, 8, 2, 320, 200),       # ~32 rows/expert: 64-row ring tiles
     (40, 8, 2, 192, 136),        # 10 rows/expert: no fused forward kernel (falls back), fused backward
     (960, 8, 2, 64, 2048),       # 240 rows/expert, about half a round of 256-row tiles: half-width tiles chosen
+    (1600, 32, 2, 64, 2048),     # 100 rows/expert and 512 wide tiles: 128x256 ring tiles
 ]
 
 
