@@ -23,7 +23,7 @@
 //   GM_S2S       row super-tiles per raster band of scatter2scatter (4: +3 % on the layer-2 shaped launches)
 //   GM_XTY       the same for groupXtY (4: 1-2 % over unbanded on all three training workloads)
 static constexpr int ROWS32_BELOW = 24, ROWS64_BELOW = 52, ROWS128_BELOW = 112, ROWS256_BELOW = 224;
-static constexpr int ROWS128W_BELOW = 136;   // 128 x 256 ring tiles for wide launches of 52..135 rows per expert
+static constexpr int ROWS128W_BELOW = 136;   // wide launches: 128 x 256 ring tiles for 52..135 rows per expert, 256 x 256 from there
 static constexpr int GM_RING = 8;
 static constexpr int STRIPE_BELOW = 1024;
 static constexpr int GM_S2S = 4;
@@ -1100,14 +1100,15 @@ static int dispatch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
     return launch_s2s<T, Tile<256, 128, 4, 2, 3>>(rest, b_tr, st);
   }
   if (avg >= ROWS256_BELOW && !half_width_wins(a)) return launch_s2s<T, Tile<256, 256, 2, 4>>(a, b_tr, st);
+  // Wide launches (enough 256-wide tile columns to fill the chip twice even with one tile row per expert, e.g.
+  // Mixtral layer 1) move half as many token rows per weight byte with 256-wide tiles as with 128-wide ones:
+  // the 256 x 256 class from 136 rows per expert on (544..832 Mixtral tokens: layer 1 -9..-11 % against the
+  // 256 x 128 ring), 128 x 256 ring tiles below (experts of about one 128-row tile: 448 tokens 518 -> 373 us,
+  // 512 tokens 520 -> 455 us).  Launches with few tile columns (Mixtral layer 2) are faster in the classes below.
+  const bool wide = (int64_t)a.E * ((a.N + (a.glu == 1 ? 127 : 255)) / (a.glu == 1 ? 128 : 256)) >= 2 * NUM_CU;
+  if (wide && avg >= ROWS128W_BELOW) return launch_s2s<T, Tile<256, 256, 2, 4>>(a, b_tr, st);
+  if (wide && avg >= ROWS64_BELOW) return launch_s2s<T, Tile<128, 256, 2, 4, 3>>(a, b_tr, st);
   // Below that the launch is a stream over the weights: ring-buffered classes, tile height by rows per expert
-  // Experts of up to about one 128-row tile each, and enough tile columns to fill the chip twice with 256-wide
-  // tiles: 128 x 256 tiles stream every weight once and carry half the token rows of the 256-row classes
-  // (Mixtral layer 1 at 448 tokens: 518 -> 373 us, at 512: 520 -> 455 us; from 144 rows per expert on and for
-  // launches with few tile columns, e.g. Mixtral layer 2, the classes below are faster).
-  if (avg >= ROWS64_BELOW && avg < ROWS128W_BELOW &&
-      (int64_t)a.E * ((a.N + (a.glu == 1 ? 127 : 255)) / (a.glu == 1 ? 128 : 256)) >= 2 * NUM_CU)
-    return launch_s2s<T, Tile<128, 256, 2, 4, 3>>(a, b_tr, st);
   if (avg >= ROWS128_BELOW) return launch_s2s<T, Tile<256, 128, 4, 2, 3>>(a, b_tr, st);
   if (avg >= ROWS32_BELOW && avg < ROWS64_BELOW) return launch_s2s<T, Tile<64, 128, 2, 2, 5>>(a, b_tr, st);
   // With one column block per wave the fused forward GLU exists only in its LDS-staged form (16-byte pieces)

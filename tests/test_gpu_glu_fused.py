@@ -24,6 +24,7 @@ SHAPES = [
     (40, 8, 2, 192, 136),        # 10 rows/expert: no fused forward kernel (falls back), fused backward
     (960, 8, 2, 64, 2048),       # 240 rows/expert, about half a round of 256-row tiles: half-width tiles chosen
     (1600, 32, 2, 64, 2048),     # 100 rows/expert and 512 wide tiles: 128x256 ring tiles
+    (2560, 32, 2, 64, 2048),     # 160 rows/expert and 512 wide tiles: 256x256 tiles below their usual threshold
 ]
 
 

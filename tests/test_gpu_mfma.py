@@ -47,6 +47,7 @@ SHAPES = [
     (2048, 32, 4, 192, 328),     # E = 32 with skew: tiny and empty experts
     (960, 8, 2, 64, 4096),       # 240 rows/expert, about half a round of 256x256 tiles: half-width tiles chosen
     (1600, 32, 2, 64, 4096),     # 100 rows/expert and 512 wide tiles: 128x256 ring tiles
+    (2560, 32, 2, 64, 4096),     # 160 rows/expert and 512 wide tiles: 256x256 tiles below their usual threshold
 ]
 
 
