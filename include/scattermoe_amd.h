@@ -50,6 +50,11 @@ enum {
 /* ABI version of the loaded library (== SMOE_ABI_VERSION it was built with). */
 int smoe_version(void);
 
+/* Hex digest of the sources (csrc/ and include/) the library was compiled from, or "unknown".  The Python loader
+ * compares it with the sources beside it and refuses a library that was built from different ones.  No counterpart
+ * in the reference (its kernels are compiled by Triton at run time). */
+const char* smoe_source_hash(void);
+
 /* Text of the last error raised on the calling thread ("" if none). Never NULL. */
 const char* smoe_last_error(void);
 
@@ -129,6 +134,8 @@ int smoe_groupXtY(const void* DY, int64_t sdym, int64_t sdyn,
  * Replaces the batched matmul `gates.unsqueeze(1) @ output_expanded` of ParallelLinear.forward
  * (scattermoe/parallel_experts.py:44-46).  Y (T*k, N) row stride sym (columns contiguous), gates (T,k)
  * strides sgt,sgk, out (T,N) row stride som.  fp32 accumulation in slot order, one rounding.
+ * gates == NULL: unit weights, i.e. the plain sum over the k slots of a token, which replaces
+ * `d_expanded_input.view(T, k, d).sum(-2)` of ParallelLinear.backward (scattermoe/parallel_experts.py:120-123).
  */
 int smoe_combine(const void* Y, int64_t sym, const void* gates, int64_t sgt, int64_t sgk, void* out, int64_t som,
                  int64_t T, int k, int64_t N, int dtype, void* stream);

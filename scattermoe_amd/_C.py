@@ -62,6 +62,11 @@ def lib_path():
     return _build.LIB_PATH
 
 
+def source_hash():
+    """Digest of the sources the loaded library was compiled from."""
+    return load().smoe_source_hash().decode()
+
+
 def load():
     """Return the loaded library, building it first if the .so is absent."""
     global _lib
@@ -78,6 +83,11 @@ def load():
                 fn.argtypes = args
             if lib.smoe_version() != 1:
                 raise RuntimeError("libscattermoe_amd.so ABI version mismatch: %d" % lib.smoe_version())
+            built_from = lib.smoe_source_hash().decode()
+            if os.path.isdir(_build.CSRC) and built_from != _build.source_hash():
+                raise RuntimeError(
+                    "libscattermoe_amd.so is stale: built from sources %s, the sources beside it are %s; "
+                    "rebuild with `python -m scattermoe_amd._build`" % (built_from, _build.source_hash()))
             _lib = lib
     return _lib
 

@@ -23,6 +23,22 @@ HIPCC_FLAGS = [
 ]
 
 
+def source_hash():
+    """sha256 over every file the library is compiled from (csrc/*.hip, csrc/*.hpp, include/*.h), first 16 hex
+    digits.  Baked into the library at build time; `_C.load` compares it with the sources it finds."""
+    import hashlib
+    inc = os.path.join(os.path.dirname(PKG_DIR), "include")
+    files = [os.path.join(CSRC, f) for f in sorted(os.listdir(CSRC)) if f.endswith((".hip", ".hpp"))]
+    if os.path.isdir(inc):
+        files += [os.path.join(inc, f) for f in sorted(os.listdir(inc)) if f.endswith(".h")]
+    h = hashlib.sha256()
+    for f in files:
+        h.update(os.path.basename(f).encode())
+        with open(f, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
 def _hipcc():
     exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(exe):
@@ -43,9 +59,12 @@ def build(verbose=False, jobs=None):
     os.makedirs(OBJ_DIR, exist_ok=True)
     objs = [os.path.join(OBJ_DIR, s.replace(".hip", ".o")) for s in SOURCES]
 
+    digest = source_hash()
+
     def one(pair):
         src, obj = pair
-        out = _run([hipcc] + HIPCC_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj])
+        extra = ['-DSMOE_SOURCE_HASH="%s"' % digest] if src == "capi.hip" else []
+        out = _run([hipcc] + HIPCC_FLAGS + extra + ["-c", os.path.join(CSRC, src), "-o", obj])
         if verbose and out.strip():
             print(out)
 

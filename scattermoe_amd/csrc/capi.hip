@@ -34,6 +34,11 @@ int smoe_version(void) { return SMOE_ABI_VERSION; }
 
 const char* smoe_last_error(void) { return g_err; }
 
+#ifndef SMOE_SOURCE_HASH
+#define SMOE_SOURCE_HASH "unknown"
+#endif
+const char* smoe_source_hash(void) { return SMOE_SOURCE_HASH; }
+
 size_t smoe_route_workspace_bytes(int64_t L, int E) {
   if (L < 0 || E <= 0) return 0;
   return route_workspace_bytes(L, E);
@@ -191,7 +196,7 @@ int smoe_combine(const void* Y, int64_t sym, const void* gates, int64_t sgt, int
   if (T < 0 || k <= 0 || N < 0) { set_error("smoe_combine: bad sizes"); return SMOE_ERR_SHAPE; }
   if (T > 0x7fffffffLL || N > 0x7fffffffLL) { set_error("smoe_combine: size beyond int32"); return SMOE_ERR_RANGE; }
   if (T == 0 || N == 0) return 0;
-  if (!Y || !gates || !out) { set_error("smoe_combine: NULL pointer"); return SMOE_ERR_NULL; }
+  if (!Y || !out) { set_error("smoe_combine: NULL pointer"); return SMOE_ERR_NULL; }
   return launch_combine(Y, sym, gates, sgt, sgk, out, som, T, k, (int)N, dtype, (hipStream_t)stream);
 }
 

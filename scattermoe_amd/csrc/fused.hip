@@ -1,6 +1,7 @@
 // HBM-bound passes around the expert GEMMs, each one read + one write instead of a library bmm or a
 // chain of elementwise launches:
-//   combine    out[t,:]  = sum_j gates[t,j] * Y[t*k+j,:]        (reference: parallel_experts.py:44-46, a bmm)
+//   combine    out[t,:]  = sum_j gates[t,j] * Y[t*k+j,:]        (reference: parallel_experts.py:44-46, a bmm;
+//                                                                 without gates: the `.sum(-2)` of :120-123)
 //   gate_grad  dg[t,j]   = <Y[t*k+j,:], dOut[t,:]>              (reference: parallel_experts.py:79, a bmm)
 //   glu_fwd    h         = act(pre[:, f:]) * pre[:, :f]          (reference: mlp.py:81-87, chunk + act + mul)
 //   glu_bwd    dpre      = [dh * act(g), dh * lin * act'(g)]     (autograd of the same expression)
@@ -39,7 +40,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const T* __restrict__ Y, i
 #pragma unroll
       for (int q = 0; q < P::n; ++q) acc[q] = 0.0f;
       for (int j = 0; j < k; ++j) {
-        const float g = to_f32(G[t * sgt + j * sgk]);
+        const float g = G ? to_f32(G[t * sgt + j * sgk]) : 1.0f;      // no gates: plain sum over the k slots
         const P x = stream_load16<P>(y0 + j * sy + (int64_t)c * P::n);
 #pragma unroll
         for (int q = 0; q < P::n; ++q) acc[q] = fmaf(g, to_f32(x.v[q]), acc[q]);
@@ -52,7 +53,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const T* __restrict__ Y, i
   } else {
     for (int n = threadIdx.x; n < N; n += 256) {
       float acc = 0.0f;
-      for (int j = 0; j < k; ++j) acc = fmaf(to_f32(G[t * sgt + j * sgk]), to_f32(y0[j * sy + n]), acc);
+      for (int j = 0; j < k; ++j) acc = fmaf(G ? to_f32(G[t * sgt + j * sgk]) : 1.0f, to_f32(y0[j * sy + n]), acc);
       O[t * so + n] = from_f32<T>(acc);
     }
   }

@@ -7,6 +7,8 @@
 //
 // One wave per token.  Lane l holds logits l, l+64, ... (at most 8 per lane, i.e. E <= 512).  Selection is k
 // rounds of a wave-wide arg-max; among equal values the lowest expert id wins.  All arithmetic in fp32.
+// Every id written is a valid expert id whatever the logits hold: a NaN logit counts as -inf, and a row without
+// any usable logit is routed as if all its logits were equal.
 #include "common.hpp"
 
 namespace smoe {
@@ -27,14 +29,18 @@ __global__ __launch_bounds__(256) void topk_softmax_kernel(const T* __restrict__
   for (int q = 0; q < ROUTER_MAX_PER_LANE; ++q) {
     const int e = q * 64 + lane;
     v[q] = e < E ? to_f32(logits[t * slt + e * sle]) : -INFINITY;
+    if (v[q] != v[q]) v[q] = -INFINITY;                        // a NaN logit never wins: its expert gets probability 0
     mx = fmaxf(mx, v[q]);
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+  const bool none = !(mx > -INFINITY);                         // no usable logit in the row: uniform probabilities
   float sum = 0.0f;
 #pragma unroll
   for (int q = 0; q < ROUTER_MAX_PER_LANE; ++q) {
-    v[q] = q * 64 + lane < E ? __expf(v[q] - mx) : -1.0f;      // -1: not a candidate (probabilities are >= 0)
+    float p = none ? 1.0f : __expf(v[q] - mx);
+    if (p != p) p = 1.0f;                                      // +inf - +inf: the logit is the maximum
+    v[q] = q * 64 + lane < E ? p : -1.0f;                      // -1: not a candidate (probabilities are >= 0)
     sum += fmaxf(v[q], 0.0f);
   }
 #pragma unroll

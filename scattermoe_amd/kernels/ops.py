@@ -95,7 +95,8 @@ class HipBackend:
         _C.require_gpu(Y, "combine")
         lib = _C.load()
         with _C.on_device(Y.device):
-            rc = lib.smoe_combine(_C.ptr(Y), Y.stride(0), _C.ptr(gates), gates.stride(0), gates.stride(1),
+            sg = (gates.stride(0), gates.stride(1)) if gates is not None else (0, 0)
+            rc = lib.smoe_combine(_C.ptr(Y), Y.stride(0), _C.ptr(gates), sg[0], sg[1],
                                   _C.ptr(out), out.stride(0), out.size(0), k, Y.size(1),
                                   _C.float_code(Y.dtype), _C.stream_ptr(Y.device))
         _C.check(rc, "smoe_combine")
@@ -274,7 +275,7 @@ def _offsets_op(eid: torch.Tensor, num_experts: int, off: torch.Tensor) -> None:
 
 
 @torch.library.custom_op("scattermoe::combine", mutates_args={"out"})
-def _combine_op(Y: torch.Tensor, gates: torch.Tensor, out: torch.Tensor, k: int) -> None:
+def _combine_op(Y: torch.Tensor, gates: Optional[torch.Tensor], out: torch.Tensor, k: int) -> None:
     _backend.combine(Y, gates, out, k)
 
 
@@ -389,6 +390,7 @@ def scatter2scatter(X, W, sorted_expert_idxs, sorted_scattered_idxs, k,
     assert L == X.size(0) * k
     assert W.dim() == 3 and W.size(1) == X.size(1)
     N = W.size(-1)
+    given = out
     if out is None:
         out = torch.empty((L, N), device=X.device, dtype=X.dtype)
     else:
@@ -399,6 +401,7 @@ def scatter2scatter(X, W, sorted_expert_idxs, sorted_scattered_idxs, k,
     else:
         _s2s_launch(out, W, X, k, sorted_expert_idxs, sorted_scattered_idxs, b,
                     x_grouped, y_grouped, expert_offsets)
+        _wrote_into(given)
     return out
 
 
@@ -474,6 +477,7 @@ def group(A, sorted_expert_idxs, coeff=None, fan_out=1, out=None):
         group_compileable(A, K, N, Y, coeff, coeff is not None, fan_out, sorted_expert_idxs)
     else:
         _group_launch(A, Y, coeff, fan_out, sorted_expert_idxs)
+        _wrote_into(out)
     return Y
 
 
@@ -504,15 +508,31 @@ def _rows_contiguous(t):
     return t if t.stride(-1) == 1 else t.contiguous()
 
 
-def combine(expanded, gates):
+def combine(expanded, gates=None):
     """out[t] = sum_j gates[t, j] * expanded[t, j]  for expanded (T, k, N) -> (T, N)
-    (the bmm of reference parallel_experts.py:44-46 as one HBM pass)."""
+    (the bmm of reference parallel_experts.py:44-46 as one HBM pass).  Without gates: the plain sum over the k
+    slots, accumulated in float32 in slot order and rounded once (the `.sum(-2)` of parallel_experts.py:120-123)."""
     T, k, N = expanded.shape
-    assert gates.shape == (T, k)
+    assert gates is None or gates.shape == (T, k)
     Y = _rows_contiguous(expanded.reshape(T * k, N))
     out = torch.empty((T, N), dtype=expanded.dtype, device=expanded.device)
-    _launch("combine", Y, gates.to(expanded.dtype), out, k)
+    _launch("combine", Y, None if gates is None else gates.to(expanded.dtype), out, k)
     return out
+
+
+def slot_sum(expanded_rows, T, k):
+    """(T*k, N) rows in slot order -> (T, N): sum over each token's k slots (one pass, no gates)."""
+    if k == 1:
+        return expanded_rows
+    return combine(expanded_rows.view(T, k, expanded_rows.size(-1)))
+
+
+def _wrote_into(t):
+    """A launch has overwritten `t` behind autograd's back: tell the version counter, so that a graph that saved
+    `t` earlier refuses to run backward a second time instead of reading the new contents (the reference gets
+    the same check from its mutating custom ops, e.g. `group` with mutates_args={'Y'}, ops.py:389)."""
+    if t is not None and not torch.compiler.is_compiling():
+        torch.autograd.graph.increment_version(t)
 
 
 def gate_grad(expanded, grad_out):

@@ -78,7 +78,7 @@ class _GatedMLP(torch.autograd.Function):
             if need_x:
                 d_exp = ops.scatter2scatter(dpre, w1.permute(0, 2, 1), eid, idx, 1, x_grouped=True, y_grouped=False,
                                             out=xg, expert_offsets=off)
-                d_x = d_exp if k == 1 else d_exp.view(x.size(0), k, d_exp.size(-1)).sum(-2)
+                d_x = ops.slot_sum(d_exp, x.size(0), k)
         return d_x, d_w1, (d_b1 if need_b1 else None), d_w2, (d_b2 if need_b2 else None), d_gates, \
             None, None, None, None, None, None, None
 

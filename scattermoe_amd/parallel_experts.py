@@ -109,7 +109,7 @@ class ParallelLinear(torch.autograd.Function):
                 X=dy, W=W.permute(0, 2, 1), k=1, x_grouped=True, y_grouped=grouped_in,
                 sorted_expert_idxs=eid, sorted_scattered_idxs=idx,
                 out=None if grouped_in else xg, expert_offsets=off)
-            d_x = d_exp if k == 1 else d_exp.view(x.size(0), k, d_exp.size(-1)).sum(-2)
+            d_x = ops.slot_sum(d_exp, x.size(0), k)
 
         return d_x, d_w, None, None, None, None, d_b, d_gates, None, None
 

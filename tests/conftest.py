@@ -24,6 +24,11 @@ def pytest_collection_modifyitems(config, items):
             item.add_marker(skip)
 
 
+def pytest_sessionfinish(session, exitstatus):
+    import _tol
+    _tol.maybe_write_report()
+
+
 @pytest.fixture
 def cpu_backend(monkeypatch):
     """Swap the HIP launch layer for the CPU oracle so that host-side logic can run without a GPU."""

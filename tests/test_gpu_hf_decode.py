@@ -227,3 +227,94 @@ def test_tiny_gpt_oss_model_end_to_end():
         torch.testing.assert_close(g_got, g_want, rtol=1e-3, atol=1e-6)
     finally:
         M.GptOssExperts.forward = patched
+
+
+def _grads(out, params, seed=9):
+    dy = torch.randn(out.shape, generator=torch.Generator().manual_seed(seed)).to(out.dtype).to(out.device)
+    return torch.autograd.grad(out, params, dy)
+
+
+@pytest.mark.parametrize("dtype,rtol,atol", [(torch.float32, 1e-4, 1e-5), (torch.bfloat16, 2e-2, 1e-2)])
+def test_granite_block_on_gpu_against_hf_original(dtype, rtol, atol):
+    """`granite_moe_forward` (reference scattermoe/utils/replace_moe.py:60-95) on the GraniteMoeHybridMoE block of
+    the installed transformers (router + experts module), forward and backward, against the block's own original
+    forward (Hugging Face's per-expert loop) run in float32 on the CPU from the same parameters."""
+    pytest.importorskip("transformers")
+    from transformers import GraniteMoeHybridConfig
+    import transformers.models.granitemoehybrid.modeling_granitemoehybrid as GR
+    from scattermoe_amd.utils import replace_moe as src
+    d, f, E, k = 128, 192, 8, 2
+    cfg = GraniteMoeHybridConfig(hidden_size=d, intermediate_size=f, num_local_experts=E, num_experts_per_tok=k,
+                                 hidden_act="silu", mamba_n_heads=4, mamba_expand=2)
+    original = getattr(GR.GraniteMoeHybridMoE.forward, "__original__", None) or GR.GraniteMoeHybridMoE.forward
+    assert original is not src.granite_moe_forward
+    g = torch.Generator().manual_seed(4)
+    ref = GR.GraniteMoeHybridMoE(cfg)
+    with torch.no_grad():
+        for prm in ref.parameters():
+            prm.copy_((torch.randn(prm.shape, generator=g) * 0.1).to(dtype).float())
+    blk = GR.GraniteMoeHybridMoE(cfg)
+    blk.load_state_dict(ref.state_dict())
+    blk = blk.to(DEV).to(dtype)
+    xin = torch.randn(3, 50, d, generator=g).to(dtype)
+    xc = xin.float().requires_grad_()
+    want = original(ref, xc)
+    xg = xin.to(DEV).requires_grad_()
+    got = src.granite_moe_forward(blk, xg)
+    assert got.shape == (3, 50, d) and got.dtype == dtype
+    # the comparison needs both sides to route alike: in bf16 the router's matmul may flip near-ties
+    same = torch.equal(blk.router(xg.detach().reshape(-1, d))[0].cpu(), ref.router(xc.detach().reshape(-1, d))[0])
+    if dtype is torch.float32:
+        assert same
+    if same:
+        _close(got, want, rtol, atol)
+        names = [n for n, _ in ref.named_parameters()]
+        for n, a, b in zip(["x"] + names, _grads(got, [xg] + list(blk.parameters())),
+                           _grads(want, [xc] + list(ref.parameters()))):
+            _close(a, b, rtol, atol)
+    else:
+        rows = (blk.router(xg.detach().reshape(-1, d))[0].cpu() == ref.router(xc.detach().reshape(-1, d))[0]).all(-1)
+        assert float(rows.float().mean()) > 0.9
+        _close(got.reshape(-1, d)[rows.to(DEV)], want.reshape(-1, d)[rows], rtol, atol)
+
+
+@pytest.mark.parametrize("dtype,rtol,atol", [(torch.float32, 1e-4, 1e-5), (torch.bfloat16, 2e-2, 1e-2)])
+def test_granite_block_of_transformers_4_on_gpu(dtype, rtol, atol):
+    """The block layout the reference patched (`router.layer`, `router.top_k`, `input_linear.weight`,
+    `output_linear.weight`, `activation`; replace_moe.py:63-93), which transformers 5.x no longer ships: a stand-in
+    with those attributes, router front end (softmax -> top-k -> renormalise in one launch) included, against the
+    oracle's per-expert form fed with `oracle.topk_softmax_ref`."""
+    from types import SimpleNamespace
+    from scattermoe_amd.utils import replace_moe as src
+    E, k, d, f = 8, 2, 128, 192
+    g = torch.Generator().manual_seed(8)
+    lw = (torch.randn(E, d, generator=g) * 0.5).to(dtype)
+    w_in = (torch.randn(E, 2 * f, d, generator=g) * 0.1).to(dtype)
+    w_out = (torch.randn(E, d, f, generator=g) * 0.1).to(dtype)
+    xin = torch.randn(4, 33, d, generator=g).to(dtype)
+    layer = torch.nn.Linear(d, E, bias=False).to(DEV).to(dtype)
+    with torch.no_grad():
+        layer.weight.copy_(lw)
+    p_in = torch.nn.Parameter(w_in.to(DEV))
+    p_out = torch.nn.Parameter(w_out.to(DEV))
+    blk = SimpleNamespace(router=SimpleNamespace(layer=layer, top_k=k, num_experts=E),
+                          input_linear=SimpleNamespace(weight=p_in), output_linear=SimpleNamespace(weight=p_out),
+                          activation=torch.nn.SiLU())
+    xg = xin.to(DEV).requires_grad_()
+    got, logits = src.granite_moe_forward(blk, xg)
+    assert got.shape == xin.shape and logits.shape == (4 * 33, E)
+    # oracle on the router logits the GPU produced (so that both sides route alike), weights rounded like the block's
+    w, sel = oracle.topk_softmax_ref(logits.detach().float().cpu(), k, True)
+    xc = xin.float().reshape(-1, d).requires_grad_()
+    gate, up = w_in.float().chunk(2, dim=1)
+    W1 = torch.cat([up, gate], 1).requires_grad_()          # the oracle's gated unit activates the SECOND half
+    W2 = w_out.float().requires_grad_()
+    want = oracle.naive_expert_forward(xc, w.to(dtype).float(), sel, W1, W2, oracle.glu(torch.nn.functional.silu))
+    _close(got.reshape(-1, d), want, rtol, atol)
+    dy = torch.randn(want.shape, generator=g).to(dtype)
+    gx, gin, gout = torch.autograd.grad(got, [xg, p_in, p_out], dy.to(DEV).view(got.shape))
+    # the oracle side keeps the routing weights constant, so compare only what does not flow through the router
+    wx, w1g, w2g = torch.autograd.grad(want, [xc, W1, W2], dy.float())
+    up_g, gate_g = w1g.chunk(2, dim=1)
+    _close(gin, torch.cat([gate_g, up_g], 1), rtol, atol)
+    _close(gout, w2g, rtol, atol)

@@ -234,3 +234,22 @@ def test_gpt_oss_glu(rows, f, dtype):
     wide = torch.zeros(rows, 2 * f + 6, dtype=dtype, device=DEV)
     wide[:, :2 * f] = pre.to(DEV)
     _close(ops.gpt_oss_glu(wide[:, :2 * f], 1.702, 7.0), want, dtype, scale=max(1.0, float(want.abs().max())))
+
+
+# ---------------------------------------------------------------------------------------------------
+# sum over the k slots of a token (the `.sum(-2)` of reference parallel_experts.py:120-123): float32 accumulation
+# in slot order, one rounding -> bit-exact against that very sequence written with torch ops
+# ---------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("T,k,N", [(1, 2, 8), (37, 4, 100), (1000, 8, 2048), (513, 3, 2880), (64, 1, 64)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_slot_sum_bit_exact(T, k, N, dtype):
+    g = torch.Generator().manual_seed(T + k + N)
+    y = torch.randn(T * k, N, generator=g).to(dtype)
+    got = ops.slot_sum(y.to(DEV), T, k)
+    acc = torch.zeros(T, N)
+    for j in range(k):
+        acc = acc + y.view(T, k, N)[:, j].float()
+    assert got.shape == (T, N) and got.dtype == dtype
+    assert torch.equal(got.cpu(), acc.to(dtype))
+    if k > 1:     # and within rounding of the library reduction the reference calls
+        _close(got, y.view(T, k, N).float().sum(-2), dtype, scale=float(k) ** 0.5)

@@ -93,3 +93,23 @@ def test_router_feeds_the_mlp():
     tw = tw / tw.sum(-1, keepdim=True)
     assert torch.equal(i, ti)
     torch.testing.assert_close(m(x, w, i), m(x, tw, ti), rtol=1e-5, atol=1e-6)
+
+
+def test_unusable_logits_still_give_valid_experts():
+    """NaN logits never win, rows without any usable logit are routed as all-equal, +inf is the maximum: every id
+    is a valid expert and every weight finite, so no row of the layer output is left unwritten downstream."""
+    E, k = 8, 2
+    nan, inf = float("nan"), float("inf")
+    logits = torch.tensor([[0.0, nan, 1.0, 2.0, nan, -1.0, 0.5, 0.25],
+                           [nan] * 8,
+                           [-inf] * 8,
+                           [0.0, inf, 1.0, 2.0, 3.0, 4.0, 5.0, 6.0],
+                           [nan, nan, nan, nan, nan, nan, nan, 3.0]])
+    w, i = ops.topk_softmax(logits.to(DEV), k, True)
+    w, i = w.cpu(), i.cpu()
+    assert bool(((i >= 0) & (i < E)).all()) and bool(torch.isfinite(w).all())
+    assert i[0].tolist() == [3, 2] and i[1].tolist() == [0, 1] and i[2].tolist() == [0, 1] and i[3, 0].item() == 1
+    assert i[4, 0].item() == 7 and abs(w[4, 0].item() - 1.0) < 1e-6
+    torch.testing.assert_close(w.sum(-1), torch.ones(5))
+    rw, ri = oracle.topk_softmax_ref(logits[:1].nan_to_num(nan=-inf), k, True)
+    torch.testing.assert_close(w[:1], rw, rtol=1e-5, atol=1e-7)

@@ -137,3 +137,33 @@ def test_product_path_refuses_cpu_tensors():
     import scattermoe_amd as sm
     with pytest.raises(RuntimeError, match="ROCm GPU only"):
         sm.flatten_sort_count(torch.tensor([[0, 1]]), 2)
+
+
+@pytest.mark.parametrize("glu", [False, True])
+def test_second_backward_over_a_consumed_graph_is_refused(cpu_backend, glu):
+    """Backward reuses the saved expert-output buffer for the grouped output gradient.  A second backward over
+    the same graph must not silently read the overwritten buffer: like the reference, whose `group` op declares
+    the buffer as mutated (scattermoe/kernels/ops.py:389), it has to raise."""
+    m, x, p, experts, dy = _case(16, 32, 24, 4, 2, False, glu)
+    y = m(x, p, experts)
+    y.backward(dy, retain_graph=True)
+    with pytest.raises(RuntimeError, match="modified by an inplace operation"):
+        y.backward(dy)
+
+
+def test_slot_sum_is_the_gateless_combine(cpu_backend):
+    ops = cpu_backend
+    y = torch.randn(5 * 3, 7)
+    assert torch.allclose(ops.slot_sum(y, 5, 3), y.view(5, 3, 7).sum(1), atol=1e-6)
+    assert ops.slot_sum(y, 15, 1) is y
+
+
+def test_stale_library_is_refused(monkeypatch):
+    """The loader compares the digest compiled into the library with the sources beside it."""
+    import scattermoe_amd._C as C
+    from scattermoe_amd import _build
+    assert C.source_hash() == _build.source_hash()
+    monkeypatch.setattr(C, "_lib", None)
+    monkeypatch.setattr(_build, "source_hash", lambda: "0" * 16)
+    with pytest.raises(RuntimeError, match="stale"):
+        C.load()
