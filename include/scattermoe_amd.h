@@ -75,6 +75,24 @@ int smoe_route(const void* expert_idxs, int idx_dtype, int64_t L, int E,
                void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * smoe_route for callers that cannot allocate: the same routing prep, same arguments and same results, but with
+ * no workspace argument.  NO COUNTERPART IN THE REFERENCE; it exists for callers that can neither call hipMalloc
+ * nor bring a workspace: code under HIP stream / graph capture, tight serving loops, harnesses that forbid
+ * allocation.  The per-chunk histograms that smoe_route keeps in the caller's workspace live in a fixed
+ * SMOE_ROUTE_STATIC_BYTES device array inside the library (one copy per GPU, held until the process ends), so the
+ * call allocates and frees nothing.  Inputs needing more than that (smoe_route_workspace_bytes(L, E) >
+ * SMOE_ROUTE_STATIC_BYTES, i.e. about ceil(L / 4096) * E > 262144) are rejected with SMOE_ERR_WORKSPACE and nothing
+ * is launched.  All calls on one GPU share the array: calls that overlap on one GPU (different streams or
+ * threads) race; calls on one stream, or otherwise ordered, are safe, and nothing has to be cleared between them.
+ * smoe_route_static_init() resolves the array's address for the CURRENT device (once per device; also done lazily
+ * by the first smoe_route_static call on a device, which therefore should not happen under stream capture).
+ */
+#define SMOE_ROUTE_STATIC_BYTES (1 << 20)
+int smoe_route_static_init(void);
+int smoe_route_static(const void* expert_idxs, int idx_dtype, int64_t L, int E,
+                      int64_t* eid_out, int64_t* idx_out, int64_t* off_out, void* stream);
+
+/*
  * Inclusive expert offsets from an already sorted id vector (off[e] = #{n : eid[n] <= e}).
  * The reference's scatter2scatter (scattermoe/kernels/ops.py:120-137) receives only eid/idx and
  * re-derives expert boundaries per 128-row block (ops.py:85-91); this library schedules

@@ -25,8 +25,11 @@ _p, _i64, _int, _sz, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctype
 _SIGNATURES = {
     "smoe_version": (_int, []),
     "smoe_last_error": (ctypes.c_char_p, []),
+    "smoe_source_hash": (ctypes.c_char_p, []),
     "smoe_route_workspace_bytes": (_sz, [_i64, _int]),
     "smoe_route": (_int, [_p, _int, _i64, _int, _p, _p, _p, _p, _sz, _p]),
+    "smoe_route_static_init": (_int, []),
+    "smoe_route_static": (_int, [_p, _int, _i64, _int, _p, _p, _p, _p]),
     "smoe_offsets_from_sorted": (_int, [_p, _i64, _int, _p, _p]),
     "smoe_scatter2scatter": (_int, [_p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64,
                                     _p, _p, _p, _i64, _i64, _i64, _int, _int, _int, _int, _int, _p]),

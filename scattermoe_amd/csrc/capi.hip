@@ -58,6 +58,20 @@ int smoe_route(const void* expert_idxs, int idx_dtype, int64_t L, int E, int64_t
   return launch_route(expert_idxs, idx_dtype, L, E, eid_out, idx_out, off_out, workspace, (hipStream_t)stream);
 }
 
+int smoe_route_static_init(void) {
+  g_err[0] = 0;
+  return route_static_init();
+}
+
+int smoe_route_static(const void* expert_idxs, int idx_dtype, int64_t L, int E, int64_t* eid_out,
+                      int64_t* idx_out, int64_t* off_out, void* stream) {
+  g_err[0] = 0;
+  if (L < 0 || E <= 0) { set_error("smoe_route_static: bad sizes L=%lld E=%d", (long long)L, E); return SMOE_ERR_SHAPE; }
+  if (L > 0x7fffffffLL) { set_error("smoe_route_static: L=%lld does not fit int32 row indexing", (long long)L); return SMOE_ERR_RANGE; }
+  if (!off_out || (L > 0 && (!expert_idxs || !eid_out || !idx_out))) { set_error("smoe_route_static: NULL pointer"); return SMOE_ERR_NULL; }
+  return launch_route_static(expert_idxs, idx_dtype, L, E, eid_out, idx_out, off_out, (hipStream_t)stream);
+}
+
 int smoe_offsets_from_sorted(const int64_t* eid, int64_t L, int E, int64_t* off_out, void* stream) {
   g_err[0] = 0;
   if (L < 0 || E <= 0) { set_error("smoe_offsets_from_sorted: bad sizes"); return SMOE_ERR_SHAPE; }

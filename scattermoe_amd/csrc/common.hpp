@@ -216,6 +216,9 @@ int launch_topk_softmax(const void* logits, int64_t slt, int64_t sle, float* w, 
 int launch_route(const void* expert_idxs, int idx_dtype, int64_t L, int E, int64_t* eid_out,
                  int64_t* idx_out, int64_t* off_out, void* ws, hipStream_t st);
 size_t route_workspace_bytes(int64_t L, int E);
+int launch_route_static(const void* expert_idxs, int idx_dtype, int64_t L, int E, int64_t* eid_out,
+                        int64_t* idx_out, int64_t* off_out, hipStream_t st);
+int route_static_init();
 int launch_offsets_from_sorted(const int64_t* eid, int64_t L, int E, int64_t* off, hipStream_t st);
 
 }  // namespace smoe

@@ -9,6 +9,7 @@
 //   scatter : stable rank inside the chunk + base           -> eid_out, idx_out
 // The result is independent of scheduling: every output position is a pure function of the input.
 #include "common.hpp"
+#include <mutex>
 
 namespace smoe {
 
@@ -234,6 +235,63 @@ static int launch_route_t(const I* ids, int64_t L, int E, int64_t* eid_out, int6
                      (size_t)kRouteWaves * E * sizeof(int), st, ids, L, E, (const int*)counts, eid_out,
                      idx_out);
   return launch_status("route_scatter_kernel");
+}
+
+// ---- routing without a caller workspace -----------------------------------------------------------------
+// The per-chunk histograms of the three-launch path live in a fixed device array instead of caller memory, for
+// callers that can neither allocate nor bring a workspace (code under stream capture, serving loops).  Each GPU
+// holds its own copy of the array at its own address; `scratch_ptr` resolves and caches that address once per
+// device.  The array keeps the previous call's contents; nothing has to start at zero, because the histogram
+// launch writes every entry the later launches read.  Calls that overlap on one GPU share the array and race.
+static __device__ __align__(256) unsigned char route_scratch[SMOE_ROUTE_STATIC_BYTES];
+
+static constexpr int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices];
+static std::mutex g_scratch_mutex;
+
+// Device address of this GPU's copy of `route_scratch` (the array's name is only a host-side handle).
+static int scratch_ptr(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    set_error("smoe_route_static: cannot identify the current device (%s)", hipGetErrorString(e));
+    return e != hipSuccess ? (int)e : SMOE_ERR_RANGE;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(route_scratch));
+    if (e != hipSuccess || p == nullptr) {
+      set_error("smoe_route_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+      return e != hipSuccess ? (int)e : SMOE_ERR_NULL;
+    }
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+
+int route_static_init() {
+  void* p = nullptr;
+  return scratch_ptr(&p);
+}
+
+int launch_route(const void* ids, int idx_dtype, int64_t L, int E, int64_t* eid_out, int64_t* idx_out,
+                 int64_t* off_out, void* ws, hipStream_t st);
+
+int launch_route_static(const void* ids, int idx_dtype, int64_t L, int E, int64_t* eid_out, int64_t* idx_out,
+                        int64_t* off_out, hipStream_t st) {
+  const size_t need = route_workspace_bytes(L, E);
+  if (need > (size_t)SMOE_ROUTE_STATIC_BYTES) {
+    set_error("smoe_route_static: L=%lld rows over E=%d experts need %zu bytes of histograms, the built-in buffer "
+              "holds %d (use smoe_route with a workspace)", (long long)L, E, need, SMOE_ROUTE_STATIC_BYTES);
+    return SMOE_ERR_WORKSPACE;
+  }
+  void* ws = nullptr;
+  if (need > 0) {
+    if (const int rc = scratch_ptr(&ws)) return rc;
+  }
+  return launch_route(ids, idx_dtype, L, E, eid_out, idx_out, off_out, ws, st);
 }
 
 int launch_route(const void* ids, int idx_dtype, int64_t L, int E, int64_t* eid_out, int64_t* idx_out,
