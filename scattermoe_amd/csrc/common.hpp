@@ -23,11 +23,14 @@ __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
 // ---- gated linear unit math (shared by the stand-alone passes and the fused GEMM epilogues) ----------------
 // Every multiplication / addition below is kept as written (no contraction into FMAs, no reassociation), so
 // that the fused epilogues and the stand-alone passes give the same bits whatever code surrounds them.
+// The reciprocal is the hardware's (v_rcp_f32, 1 ulp) rather than a correctly rounded division: the epilogues of
+// the fused launches spend their time in this function (a division is about ten instructions), and every result
+// is rounded to a 16-bit type or compared at 1e-4 afterwards.
 __device__ __forceinline__ float sigmoidf_(float x) {
 #pragma clang fp contract(off) reassociate(off)
   const float e = __expf(-x);
   const float d = 1.0f + e;
-  return 1.0f / d;
+  return __builtin_amdgcn_rcpf(d);
 }
 // act & 1 selects which half of `pre` is the activated (gate) half: 0 = second half (GLUMLP of the reference),
 // 1 = first half (the Hugging Face `act(gate) * up` convention).  The activation itself is SiLU.
@@ -62,6 +65,21 @@ __device__ __forceinline__ float glu_dgat(int act, float dh, float gat, float li
   const float t = dh * lin;
   const float d = act_df(act, gat);
   return t * d;
+}
+
+// both gradients at once (one sigmoid); same operations in the same order as glu_dlin and glu_dgat
+__device__ __forceinline__ void glu_grad(int act, float dh, float gat, float lin, float& d_lin, float& d_gat) {
+#pragma clang fp contract(off) reassociate(off)
+  (void)act;
+  const float s = sigmoidf_(gat);
+  const float a0 = gat * s;
+  d_lin = dh * a0;
+  const float t = dh * lin;
+  const float a = 1.0f - s;
+  const float b = gat * a;
+  const float c = 1.0f + b;
+  const float d = s * c;
+  d_gat = t * d;
 }
 
 // gated unit of the gpt-oss experts over one (gate, up) pair and its gradient (clamped inputs pass no gradient)

@@ -615,7 +615,9 @@ __device__ __forceinline__ void epilogue_glu_bwd(const f32x16 (&acc)[TL::FM][TL:
         for (int e = 0; e < 4; ++e) {
           const float dv = to_f32(from_f32<T>(acc[i][j][g * 4 + e]));
           const float lin = to_f32(gf ? p2[e] : p1[e]), gat = to_f32(gf ? p1[e] : p2[e]);
-          const T d_lin = from_f32<T>(glu_dlin(a.act, dv, gat)), d_gat = from_f32<T>(glu_dgat(a.act, dv, gat, lin));
+          float f_lin, f_gat;
+          glu_grad(a.act, dv, gat, lin, f_lin, f_gat);
+          const T d_lin = from_f32<T>(f_lin), d_gat = from_f32<T>(f_gat);
           o1[e] = gf ? d_gat : d_lin;
           o2[e] = gf ? d_lin : d_gat;
         }
@@ -742,7 +744,9 @@ __device__ __forceinline__ void epilogue_glu_bwd_staged(const f32x16 (&acc)[TL::
       for (int e = 0; e < 8; ++e) {
         const float dv = to_f32(dh[u][e]);
         const float lin = to_f32(gf ? p2[u][e] : p1[u][e]), gat = to_f32(gf ? p1[u][e] : p2[u][e]);
-        const T d_lin = from_f32<T>(glu_dlin(a.act, dv, gat)), d_gat = from_f32<T>(glu_dgat(a.act, dv, gat, lin));
+        float f_lin, f_gat;
+          glu_grad(a.act, dv, gat, lin, f_lin, f_gat);
+          const T d_lin = from_f32<T>(f_lin), d_gat = from_f32<T>(f_gat);
         o1[e] = gf ? d_gat : d_lin;
         o2[e] = gf ? d_lin : d_gat;
       }
