@@ -20,12 +20,75 @@ os.environ.setdefault("SCATTERMOE_NO_HF_PATCH", "1")
 PEAK_BF16_TFLOPS = 2500.0        # MI355X dense bf16 MFMA peak
 PEAK_HBM_GBS = 8000.0
 
-# HBM bytes moved per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (KiB per dispatch, scaled by a copy kernel of known size); None until measured for a workload.
-# c2: average over the two products of the dominant kernel in a step (layer-1 forward with the gated linear unit
-# in its epilogue 21.33 GB, layer-2 forward 7.49 GB; see profiles/s2s_mfma_c2_l1fwd_counters.md for the commands
-# and raw counter values).
-MEASURED_TRAFFIC = {"c2": 14.41e9}
+
+
+def measured_traffic(workload, source_hash):
+    """HBM-side bytes per launch of the dominant kernel, from profiles/<workload>_traffic.json - the record a
+    rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE session of this benchmark leaves (profiles/README.md has the commands).
+    The record names the kernel sources it was measured on; for any other sources the figure would be a guess,
+    so None is returned."""
+    path = os.path.join(ROOT, "profiles", "%s_traffic.json" % workload)
+    try:
+        with open(path) as f:
+            rec = json.load(f)
+    except (OSError, ValueError):
+        return None, None
+    if rec.get("source_hash") != source_hash:
+        return None, "profiles/%s_traffic.json was measured on kernel sources %s, this library is %s" % (
+            workload, rec.get("source_hash"), source_hash)
+    return rec.get("bytes_per_launch"), "profiles/%s_traffic.json (%s)" % (workload, rec.get("command", ""))
+
+
+def traffic_record(args):
+    """HBM-side bytes per product of the dominant kernel from four rocprofv3 --pmc runs (one counter each):
+    DIR/fetch, DIR/write = FETCH_SIZE / WRITE_SIZE over `bench.py --workload W --no-cpu`, DIR/fetch_copy, DIR/write_copy
+    = the same counters over `bench.py --profile-kernel copy` (256 MiB read + 256 MiB written per launch), which give
+    the factor from counter units to KiB.  The dominant kernel's products are the scatter2scatter launches with
+    K-contiguous weights (kernel instantiations with B_TR = false); a product split over two launches counts once."""
+    import csv
+    import glob
+    import subprocess
+
+    def rows(sub):
+        out = []
+        for f in glob.glob(os.path.join(args.traffic_record, sub, "**", "*counter_collection.csv"), recursive=True):
+            out += list(csv.DictReader(open(f)))
+        return out
+
+    def per_launch(sub, counter, want):
+        v = [float(r["Counter_Value"]) for r in rows(sub) if r["Counter_Name"] == counter and want(r["Kernel_Name"])]
+        return v
+
+    copy_kib = 256.0 * 1024
+    is_copy = lambda n: "copyBuffer" in n
+    f_copy = per_launch("fetch_copy", "FETCH_SIZE", is_copy)
+    w_copy = per_launch("write_copy", "WRITE_SIZE", is_copy)
+    f_factor = copy_kib / (sum(f_copy) / len(f_copy))
+    w_factor = copy_kib / (sum(w_copy) / len(w_copy))
+    # B_TR = false instantiations of the scatter2scatter MFMA kernel, any tile class
+    dominant = lambda n: "s2s_mfma_kernel" in n and ("Lb0EEEv" in n or "false>" in n)
+    fetch = per_launch("fetch", "FETCH_SIZE", dominant)
+    write = per_launch("write", "WRITE_SIZE", dominant)
+    steps = args.steps + args.warmup
+    products_per_step = 2
+    n_products = steps * products_per_step
+    fetch_b = sum(fetch) * f_factor * 1024 / n_products
+    write_b = sum(write) * w_factor * 1024 / n_products
+    sys.path.insert(0, ROOT)
+    from scattermoe_amd import _build
+    try:
+        commit = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], capture_output=True, text=True).stdout.strip()
+    except OSError:
+        commit = ""
+    print(json.dumps({
+        "workload": args.workload, "kernel": "s2s_mfma_kernel, products with K-contiguous weights (layer-1 and layer-2 forward)",
+        "bytes_per_launch": round(fetch_b + write_b), "fetch_bytes": round(fetch_b), "write_bytes": round(write_b),
+        "launches_counted": {"fetch": len(fetch), "write": len(write)}, "products": n_products,
+        "factor_to_kib": {"FETCH_SIZE": round(f_factor, 4), "WRITE_SIZE": round(w_factor, 4)},
+        "source_hash": _build.source_hash(), "commit": commit,
+        "command": "rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE --output-format csv -- python3 bench.py --workload %s --steps %d "
+                   "--warmup %d --no-cpu; same counters over python3 bench.py --profile-kernel copy --steps 10"
+                   % (args.workload, args.steps, args.warmup)}, indent=1))
 
 
 def parse():
@@ -42,28 +105,35 @@ def parse():
     ap.add_argument("--profile-kernel", default="",
                     help="run ONLY one kernel of the workload `steps` times (for rocprofv3 --pmc): "
                          "l1fwd | l2fwd | l1dx | l2dx | l1dw | l2dw | copy (a 256 MiB device copy of known size)")
+    ap.add_argument("--traffic-record", default="", metavar="DIR",
+                    help="no GPU work: read the rocprofv3 --pmc csv files under DIR/{fetch,write,fetch_copy,write_copy} "
+                         "(FETCH_SIZE / WRITE_SIZE over a run of this benchmark and over `--profile-kernel copy`) and "
+                         "print the traffic record that belongs into profiles/<workload>_traffic.json")
     return ap.parse_args()
 
 
 class TimedBackend:
-    """Wraps the launch layer and brackets every scatter2scatter launch with events on the launch stream."""
+    """Wraps the launch layer and brackets every expert-GEMM launch (scatter2scatter, groupXtY) with events on the
+    launch stream.  Records: (start, stop, algorithmic FLOP, weights K-contiguous? (None for groupXtY), product name)."""
 
-    def __init__(self, inner, torch):
+    def __init__(self, inner, torch, cfg):
         self.inner, self.torch, self.records, self.on = inner, torch, [], False
+        self.l1_dw_shape = ((2 if cfg.glu else 1) * cfg.f, cfg.d)     # (columns of dY, columns of X) of the layer-1 dW
 
     def __getattr__(self, name):
         return getattr(self.inner, name)
 
     def s2s(self, X, W, b, Y, eid, idx, off, k, x_grouped, y_grouped):
-        if not self.on:
-            return self.inner.s2s(X, W, b, Y, eid, idx, off, k, x_grouped, y_grouped)
-        a, c = self.torch.cuda.Event(enable_timing=True), self.torch.cuda.Event(enable_timing=True)
-        a.record()
-        self.inner.s2s(X, W, b, Y, eid, idx, off, k, x_grouped, y_grouped)
-        c.record()
-        self.records.append((a, c, 2.0 * eid.numel() * X.size(1) * Y.size(1), W.stride(1) == 1))
+        name = ("l1_fwd" if not x_grouped else "l2_fwd") if W.stride(1) == 1 else ("l1_dx" if not y_grouped else "l2_dx")
+        return self._timed(lambda: self.inner.s2s(X, W, b, Y, eid, idx, off, k, x_grouped, y_grouped) is None,
+                           2.0 * eid.numel() * X.size(1) * Y.size(1), W.stride(1) == 1, name)
 
-    def _timed(self, fn, flops, k_contig):
+    def xty(self, DY, X, DW, Db, off, E):
+        name = "l1_dw" if (DY.size(1), X.size(1)) == self.l1_dw_shape else "l2_dw"
+        return self._timed(lambda: self.inner.xty(DY, X, DW, Db, off, E) is None,
+                           2.0 * DY.size(0) * X.size(1) * DY.size(1), None, name)
+
+    def _timed(self, fn, flops, k_contig, name):
         if not self.on:
             return fn()
         a, c = self.torch.cuda.Event(enable_timing=True), self.torch.cuda.Event(enable_timing=True)
@@ -71,17 +141,17 @@ class TimedBackend:
         ok = fn()
         c.record()
         if ok:
-            self.records.append((a, c, flops, k_contig))
+            self.records.append((a, c, flops, k_contig, name))
         return ok
 
     # the fused GEMM + gated-linear-unit launches are launches of the same kernel (scatter2scatter FLOPs only)
     def s2s_glu(self, X, W, b, pre, h, eid, idx, off, k, x_grouped, act):
         return self._timed(lambda: self.inner.s2s_glu(X, W, b, pre, h, eid, idx, off, k, x_grouped, act),
-                           2.0 * eid.numel() * X.size(1) * W.size(2), W.stride(1) == 1)
+                           2.0 * eid.numel() * X.size(1) * W.size(2), W.stride(1) == 1, "l1_fwd")
 
     def s2s_glu_bwd(self, DY, W, pre, dpre, eid, idx, off, act):
         return self._timed(lambda: self.inner.s2s_glu_bwd(DY, W, pre, dpre, eid, idx, off, act),
-                           2.0 * eid.numel() * DY.size(1) * W.size(2), W.stride(1) == 1)
+                           2.0 * eid.numel() * DY.size(1) * W.size(2), W.stride(1) == 1, "l2_dx")
 
 
 def cpu_baseline(cfg, tokens, torch):
@@ -196,6 +266,9 @@ def decode_line(args, cfg, torch):
 
 def main():
     args = parse()
+    if args.traffic_record:
+        traffic_record(args)
+        return
     if args.gpus != 1:
         print("bench.py: this build measures ONE GPU; --gpus %d is not supported "
               "(no collective or multi-GPU code exists in this path)" % args.gpus, file=sys.stderr)
@@ -222,24 +295,19 @@ def main():
         decode_line(args, cfg, torch)
         return
 
-    # synthetic inputs, generated on the device with a fixed seed; resident before timing starts
-    g = torch.Generator(device=dev).manual_seed(0)
-    logits = torch.randn(cfg.T, cfg.E, generator=g, device=dev)
-    if cfg.zipf_beta:
-        logits = logits - cfg.zipf_beta * 1.2 * torch.log(torch.arange(1, cfg.E + 1, device=dev).float())
-    p, experts = torch.topk(torch.softmax(logits, -1), cfg.k)
-    p = (p / p.sum(-1, keepdim=True)).to(dtype).requires_grad_()
-    x = torch.randn(cfg.T, cfg.d, generator=g, device=dev).to(dtype).requires_grad_()
-    dy = torch.randn(cfg.T, cfg.d, generator=g, device=dev).to(dtype)
-    cls = GLUMLP if cfg.glu else MLP
-    with torch.device(dev):
-        m = cls(cfg.d, cfg.f, cfg.E, cfg.k, bias=cfg.bias, activation=nn.SiLU() if cfg.glu else nn.GELU()).to(dtype)
-    if cfg.bias:
-        nn.init.normal_(m.experts.bias, std=0.02)
-        nn.init.normal_(m.output_experts.bias, std=0.02)
+    # synthetic inputs, resident in HBM before timing starts.  Router logits (hence routing and gates), X and dY are
+    # drawn on the CPU (seed 0, the draw order of tests/_inputs.make_inputs: the tensors the full-shape parity tests
+    # use); the weights are drawn on the device (seed 1, tests/_inputs.make_module)
+    from _inputs import make_inputs, make_module
+    t = make_inputs(cfg, weights=False)
+    experts = t["experts"].to(dev)
+    p = t["p"].to(dtype).to(dev).requires_grad_()
+    x = t["x"].to(dtype).to(dev).requires_grad_()
+    dy = t["dy"].to(dtype).to(dev)
+    m = make_module(cfg, dev)
     leaves = [x, p] + list(m.parameters())
 
-    timed = TimedBackend(ops._backend, torch)
+    timed = TimedBackend(ops._backend, torch, cfg)
     ops._backend = timed
 
     def step():
@@ -265,14 +333,22 @@ def main():
     tflops = flops_step / (ms * 1e-3) / 1e12
 
     # dominant kernel: the MFMA scatter2scatter (forward flavour: weights with contiguous contraction axis)
-    fwd = [(a.elapsed_time(c), fl) for a, c, fl, kc in timed.records if kc]
-    allk = [(a.elapsed_time(c), fl) for a, c, fl, kc in timed.records]
+    fwd = [(a.elapsed_time(c), fl) for a, c, fl, kc, _ in timed.records if kc]
+    allk = [(a.elapsed_time(c), fl) for a, c, fl, kc, _ in timed.records if kc is not None]
     sel = fwd if fwd else allk
+    # every product of the step by itself: TFLOP/s over its algorithmic 2 L K N, averaged over the timed steps
+    products = {}
+    for a, c, fl, _, name in timed.records:
+        ms_, fl_ = products.get(name, (0.0, 0.0))
+        products[name] = (ms_ + a.elapsed_time(c), fl_ + fl)
+    products = {n: {"ms": round(v[0] / args.steps, 4), "tflops": round(v[1] / v[0] / 1e9, 1),
+                    "frac": round(v[1] / v[0] / 1e9 / PEAK_BF16_TFLOPS, 4)} for n, v in sorted(products.items())}
     k_ms = sum(t for t, _ in sel) / len(sel)
     k_fl = sum(fl for _, fl in sel) / len(sel)
     achieved = k_fl / (k_ms * 1e-3) / 1e12
+    traffic, traffic_src = measured_traffic(cfg.name, _C.source_hash())
     roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": MEASURED_TRAFFIC.get(cfg.name),
+                "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": traffic, "traffic_source": traffic_src,
                 "kernel": "s2s_mfma_kernel (scatter2scatter products with K-contiguous weights; a product of a few "
                           "rounds of tiles plus a remainder runs as two launches and is timed as one)",
                 "launches_per_step": len(sel) // args.steps, "avg_launch_ms": round(k_ms, 4),
@@ -289,6 +365,10 @@ def main():
             "tokens": cfg.T, "rows": L},
         "tflops": round(tflops, 1), "frac_of_bf16_mfma_peak": round(tflops / PEAK_BF16_TFLOPS, 4),
         "roofline": roofline,
+        "products": products,
+        "inputs": "router logits, X, dY: CPU generator seed 0 (tests/_inputs.make_inputs order); weights: device "
+                  "generator seed 1, N(0, 0.02) (tests/_inputs.make_module)",
+        "library_sources": _C.source_hash(),
     }
     if not args.no_cpu:
         tokens = args.cpu_tokens or max(64, cfg.T // 16)

@@ -51,3 +51,21 @@ def make_inputs(cfg, seed=0, weights=True):
             out["b2"] = torch.randn(cfg.E, cfg.d, generator=g) * 0.02
     out["dy"] = torch.randn(cfg.T, cfg.d, generator=g)
     return out
+
+
+def make_module(cfg, device, seed=1):
+    """The module of a configuration with weights (and biases) drawn N(0, 0.02) on `device` from a device generator:
+    the draw that the full-shape GPU tests and bench.py share (drawing up to 5.6e9 normal numbers on the host takes
+    longer than everything else they do)."""
+    from torch import nn
+    from scattermoe_amd.mlp import GLUMLP, MLP
+    g = torch.Generator(device=device).manual_seed(seed)
+    with torch.device(device):
+        if cfg.glu:
+            m = GLUMLP(cfg.d, cfg.f, cfg.E, cfg.k, bias=cfg.bias).to(cfg.dtype)
+        else:
+            m = MLP(cfg.d, cfg.f, cfg.E, cfg.k, bias=cfg.bias, activation=nn.GELU()).to(cfg.dtype)
+    with torch.no_grad():
+        for prm in m.parameters():
+            prm.copy_((torch.randn(prm.shape, generator=g, device=device) * 0.02).to(cfg.dtype))
+    return m

@@ -20,9 +20,8 @@ import torch
 from torch import nn
 
 import oracle
-from _inputs import CONFIGS, make_inputs
+from _inputs import CONFIGS, make_inputs, make_module
 from _tol import check
-from scattermoe_amd.mlp import GLUMLP
 from scattermoe_amd.parallel_experts import flatten_sort_count
 
 pytestmark = pytest.mark.gpu
@@ -31,13 +30,7 @@ BF = torch.bfloat16
 
 
 def _module(cfg):
-    g = torch.Generator(device=DEV).manual_seed(1)
-    with torch.device(DEV):
-        m = GLUMLP(cfg.d, cfg.f, cfg.E, cfg.k, bias=cfg.bias).to(cfg.dtype)
-    with torch.no_grad():
-        for prm in m.parameters():
-            prm.copy_((torch.randn(prm.shape, generator=g, device=DEV) * 0.02).to(cfg.dtype))
-    return m
+    return make_module(cfg, DEV)
 
 
 def _step(cfg):
