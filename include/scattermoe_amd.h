@@ -148,6 +148,21 @@ int smoe_groupXtY(const void* DY, int64_t sdym, int64_t sdyn,
                   int dtype, void* stream);
 
 /*
+ * smoe_groupXtY with X given as the (L / fan_out, K) matrix its grouped rows come from: grouped row r of X is
+ * X[idx[r] / fan_out].  Replaces the pair `group(x, sorted_scattered_idxs, fan_out=k)` + `group_bwd_W(...)` of
+ * ParallelLinear.backward (scattermoe/parallel_experts.py:95-107: the gathered copy of x exists only to feed the
+ * weight gradient), saving one write and one read of an (L, K) matrix.  Same results as grouping first.
+ * Returns SMOE_ERR_UNSUPPORTED (nothing launched) for float32 or operands the MFMA kernels do not take; the caller
+ * then groups X and calls smoe_groupXtY.
+ */
+int smoe_groupXtY_gathered(const void* DY, int64_t sdym, int64_t sdyn,
+                           const void* X, int64_t sxm, int64_t sxk, const int64_t* idx, int fan_out,
+                           void* DW, int64_t sdwe, int64_t sdwk, int64_t sdwn,
+                           void* Db, int64_t sdbe, int64_t sdbn,
+                           const int64_t* off, int64_t L, int64_t K, int64_t N, int E,
+                           int dtype, void* stream);
+
+/*
  * Gate-weighted sum of the k expert outputs of each token:  out[t,:] = sum_j gates[t,j] * Y[t*k+j,:].
  * Replaces the batched matmul `gates.unsqueeze(1) @ output_expanded` of ParallelLinear.forward
  * (scattermoe/parallel_experts.py:44-46).  Y (T*k, N) row stride sym (columns contiguous), gates (T,k)

@@ -36,6 +36,8 @@ _SIGNATURES = {
     "smoe_group": (_int, [_p, _i64, _i64, _p, _p, _i64, _i64, _p, _i64, _i64, _int, _int, _p]),
     "smoe_groupXtY": (_int, [_p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _i64,
                              _p, _i64, _i64, _i64, _int, _int, _p]),
+    "smoe_groupXtY_gathered": (_int, [_p, _i64, _i64, _p, _i64, _i64, _p, _int, _p, _i64, _i64, _i64, _p, _i64, _i64,
+                                      _p, _i64, _i64, _i64, _int, _int, _p]),
     "smoe_combine": (_int, [_p, _i64, _p, _i64, _i64, _p, _i64, _i64, _int, _i64, _int, _p]),
     "smoe_gate_grad": (_int, [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _int, _i64, _int, _p]),
     "smoe_glu_fwd": (_int, [_p, _i64, _p, _i64, _i64, _i64, _int, _int, _p]),

@@ -203,6 +203,24 @@ int smoe_groupXtY(const void* DY, int64_t sdym, int64_t sdyn, const void* X, int
   return launch_xty_generic(a, dtype, (hipStream_t)stream);
 }
 
+int smoe_groupXtY_gathered(const void* DY, int64_t sdym, int64_t sdyn, const void* X, int64_t sxm, int64_t sxk,
+                           const int64_t* idx, int fan_out, void* DW, int64_t sdwe, int64_t sdwk, int64_t sdwn,
+                           void* Db, int64_t sdbe, int64_t sdbn, const int64_t* off, int64_t L, int64_t K, int64_t N,
+                           int E, int dtype, void* stream) {
+  g_err[0] = 0;
+  if (!dtype_ok(dtype)) { set_error("smoe_groupXtY_gathered: unknown dtype %d", dtype); return SMOE_ERR_DTYPE; }
+  if (L < 0 || K < 0 || N < 0 || E <= 0 || fan_out <= 0) { set_error("smoe_groupXtY_gathered: bad sizes"); return SMOE_ERR_SHAPE; }
+  if (L > 0x7fffffffLL || K > 0x7fffffffLL || N > 0x7fffffffLL) { set_error("smoe_groupXtY_gathered: size beyond int32"); return SMOE_ERR_RANGE; }
+  if (K == 0 || N == 0) return 0;
+  if (!DW || !off || (L > 0 && (!DY || !X || !idx))) { set_error("smoe_groupXtY_gathered: NULL pointer"); return SMOE_ERR_NULL; }
+  XtYArgs a{DY, sdym, sdyn, X, sxm, sxk, DW, sdwe, sdwk, sdwn, Db, sdbe, sdbn, off, (int)L, (int)K, (int)N, E};
+  a.idx = idx;
+  a.fan_out = fan_out;
+  int rc = 0;
+  if (try_xty_mfma(a, dtype, (hipStream_t)stream, rc)) return rc;
+  return SMOE_ERR_UNSUPPORTED;       // only the MFMA kernels gather; the caller groups X itself and calls smoe_groupXtY
+}
+
 int smoe_combine(const void* Y, int64_t sym, const void* gates, int64_t sgt, int64_t sgk, void* out, int64_t som,
                  int64_t T, int k, int64_t N, int dtype, void* stream) {
   g_err[0] = 0;

@@ -179,6 +179,10 @@ struct XtYArgs {
   void* Db; int64_t sdbe, sdbn;
   const int64_t* off;
   int L, K, N, E;
+  // X is the (L / fan_out, K) matrix the grouped rows would be gathered from: grouped row r = X[idx[r] / fan_out]
+  // (MFMA path only); NULL: X holds the L grouped rows themselves
+  const int64_t* idx = nullptr;
+  int fan_out = 1;
 };
 
 struct GroupArgs {

@@ -28,6 +28,7 @@ static constexpr int GM_RING = 8;
 static constexpr int STRIPE_BELOW = 1024;
 static constexpr int GM_S2S = 4;
 static constexpr int GM_XTY = 4;
+static constexpr int XTY_GATHER_MAX_N = 6144;   // widest dY for which groupXtY gathers the rows of X itself
 #include <type_traits>
 #include <algorithm>
 #include <math.h>
@@ -184,13 +185,23 @@ struct DirectOp {
     const int row = base + (l & 31);
     return lds_read16(tile + row * 128 + (((2 * ks + (l >> 5)) ^ direct_swz(row)) << 4));
   }
+  // only operands that gather their contraction rows have anything to do here (see TransOp)
+  __device__ __forceinline__ void fetch_rows(int, int) {}
+  __device__ __forceinline__ void stage_rows(int) {}
+  __device__ __forceinline__ void take_rows(int) {}
 };
 
 // ---- operand with strided contraction axis: LDS tile [64][EXT], read transposed --------------------------
 // Row kr of the tile is EXT*2 bytes = G granules of 64 B (32 columns).  A ds_read_b64_tr_b16 phase touches
 // one granule column in 4 consecutive rows; storing granule g of row kr at position g ^ (kr & 3) spreads
 // those 4 accesses over all 64 banks.
-template <int EXT, int NT, bool STREAM = false>
+// GATHER: the contraction rows are not consecutive in memory but picked through an index vector (row r of the
+// operand is row rows[r] / fan of the source matrix).  The 64 rows of a slice are looked up once per workgroup, not
+// once per thread (vector-ALU work in this loop comes straight out of the matrix pipe's time): thread t < 64 fetches
+// the index of row t one slice ahead (`fetch_rows`, an ordinary load that the main loop's wait covers), turns it into
+// a byte offset and puts it into LDS before the loop's barrier (`stage_rows`); after the barrier every thread picks
+// the offsets of its own load slots up from there (`take_rows`).
+template <int EXT, int NT, bool STREAM = false, bool GATHER = false>
 struct TransOp {
   static constexpr int CPR = EXT / 8;                  // 16-byte pieces per contraction row
   static constexpr int PIECES = 64 * CPR;
@@ -201,9 +212,18 @@ struct TransOp {
   static_assert(PIECES % NT == 0 && EXT % 128 == 0, "unsupported transposed tile width");
   const char* base;    // wave-uniform global address of (contraction 0, column 0 of the tile)
   unsigned off[R];     // byte offset of this thread's piece of load slot j within the first slice
+                       // (GATHER: within the slice that is issued next)
   int rot = 0;         // load slot j carries round (j + rot) % R (see DirectOp)
   __device__ __forceinline__ int rnd(int j) const { const int r = j + rot; return r >= R ? r - R : r; }
   int64_t ld;          // bytes between contraction rows
+  // GATHER only
+  const int64_t* rows; // wave-uniform: index vector, already offset to the first contraction row
+  unsigned fan;
+  unsigned colb[R];    // byte offset of this thread's piece inside its contraction row
+  unsigned next_row;   // thread t < 64: index of contraction row t of the slice after the one being issued
+  unsigned* srow;      // LDS, [2][64]: byte offsets of the rows of the slice to be issued next, by slice parity
+  // contraction row inside a slice that load slot j of this thread carries
+  __device__ __forceinline__ int slot_row(int j) const { return (rnd(j) * NT + (int)threadIdx.x) / CPR; }
   // columns >= valid_cols are clamped to column 0 (they only feed outputs that are never stored)
   __device__ __forceinline__ void init(const char* b, int64_t ld_bytes, int valid_cols) {
     init_cols(b, ld_bytes, [&](int tc) { return tc < valid_cols ? tc : 0; });
@@ -220,11 +240,50 @@ struct TransOp {
       const int p = rnd(j) * NT + t;
       const int kr = p / CPR, phys = p % CPR;
       const int cc = ((((phys >> 2) ^ (kr & 3)) << 2) | (phys & 3));      // logical 16-byte piece of the row
-      off[j] = (unsigned)(kr * ld_bytes) + (unsigned)col_of(cc * 8) * 2;
+      if constexpr (GATHER) colb[j] = (unsigned)col_of(cc * 8) * 2;
+      else off[j] = (unsigned)(kr * ld_bytes) + (unsigned)col_of(cc * 8) * 2;
+    }
+  }
+  // GATHER: `b` is (row 0, column 0 of the tile) of the SOURCE matrix, `r` the index vector at the operand's first
+  // contraction row, `klen` the number of contraction rows, `lds_rows` 2 x 64 words of LDS.  Ends with the first
+  // slice's offsets taken (one workgroup barrier inside).
+  __device__ __forceinline__ void init_gather(const char* b, int64_t ld_bytes, int valid_cols, const int64_t* r,
+                                              int fan_out, int klen, unsigned* lds_rows) {
+    rows = (const int64_t*)make_uniform((const char*)r);
+    fan = (unsigned)fan_out;
+    srow = lds_rows;
+    init(b, ld_bytes, valid_cols);
+    fetch_rows(0, klen);
+    stage_rows(0);
+    __syncthreads();
+    take_rows(0);
+  }
+  // index of row t of the slice at contraction k0 (rows past the end repeat the last row: their data is zeroed in LDS)
+  __device__ __forceinline__ void fetch_rows(int k0, int klen) {
+    if constexpr (GATHER) {
+      if (wave_uniform_id() == 0) {
+        int r = k0 + (int)threadIdx.x;
+        r = r < klen ? r : klen - 1;
+        next_row = r >= 0 ? (unsigned)rows[r] : 0u;
+      }
+    }
+  }
+  // before the barrier of the iteration that issues slice number `slice`
+  __device__ __forceinline__ void stage_rows(int slice) {
+    if constexpr (GATHER) {
+      if (wave_uniform_id() == 0) srow[(slice & 1) * 64 + threadIdx.x] = (unsigned)((int64_t)(next_row / fan) * ld);
+    }
+  }
+  // after that barrier
+  __device__ __forceinline__ void take_rows(int slice) {
+    if constexpr (GATHER) {
+#pragma unroll
+      for (int j = 0; j < R; ++j) off[j] = srow[(slice & 1) * 64 + slot_row(j)] + colb[j];
     }
   }
   __device__ __forceinline__ void issue_one(unsigned tile, int k0, int j) const {
-    load_to_lds16<STREAM>(base + (int64_t)k0 * ld, off[j], tile + wave_uniform_id() * 1024 + rnd(j) * NT * 16);
+    if constexpr (GATHER) load_to_lds16<STREAM>(make_uniform(base), off[j], tile + wave_uniform_id() * 1024 + rnd(j) * NT * 16);
+    else load_to_lds16<STREAM>(base + (int64_t)k0 * ld, off[j], tile + wave_uniform_id() * 1024 + rnd(j) * NT * 16);
   }
   __device__ __forceinline__ void issue(unsigned tile, int k0) const {
 #pragma unroll
@@ -233,10 +292,14 @@ struct TransOp {
   // Partial last slice: contraction rows past `kend` are fetched from row 0 of the slice (always valid
   // memory) and overwritten with zeros by the same thread once its loads have landed.
   __device__ __forceinline__ void issue_tail_one(unsigned tile, int k0, int kend, int j) const {
-    const int kr = (rnd(j) * NT + (int)threadIdx.x) / CPR;
-    const bool ok = k0 + kr < kend;
-    load_to_lds16<STREAM>(base + (int64_t)k0 * ld, ok ? off[j] : off[j] - (unsigned)(kr * ld),
-                  tile + wave_uniform_id() * 1024 + rnd(j) * NT * 16);
+    if constexpr (GATHER) {
+      issue_one(tile, k0, j);          // rows past the end already point at the last valid row
+    } else {
+      const int kr = slot_row(j);
+      const bool ok = k0 + kr < kend;
+      load_to_lds16<STREAM>(base + (int64_t)k0 * ld, ok ? off[j] : off[j] - (unsigned)(kr * ld),
+                    tile + wave_uniform_id() * 1024 + rnd(j) * NT * 16);
+    }
   }
   __device__ __forceinline__ void issue_tail(unsigned tile, int k0, int kend) const {
 #pragma unroll
@@ -304,7 +367,7 @@ struct Tile {
 // If `rowsum`, rs[i] additionally accumulates, per lane, the sum of the lane's own 8 contraction elements of
 // A-fragment i; adding lanes l and l+32 afterwards gives the sum over the contraction of A row l%32.
 template <typename T, class TL, class AOp, class BOp, bool CAN_ROWSUM>
-__device__ __forceinline__ void mainloop(const AOp& A, const BOp& B, int klen, char* lds, bool rowsum,
+__device__ __forceinline__ void mainloop(AOp& A, BOp& B, int klen, char* lds, bool rowsum,
                                          f32x16 (&acc)[TL::FM][TL::FN], float (&rs)[TL::FM]) {
   constexpr int STAGE = AOp::LDS_BYTES + BOp::LDS_BYTES;
   const int wave = threadIdx.x >> 6;
@@ -315,6 +378,8 @@ __device__ __forceinline__ void mainloop(const AOp& A, const BOp& B, int klen, c
   const unsigned lds_u = lds_address(lds);
   if (nfull > 0) issue_slice(A, B, lds_u, 0);
   else if (tail) issue_slice_tail(A, B, lds_u, 0, klen);
+  A.fetch_rows(BK, klen);            // gathered operands: row indices of the slice after the one just issued
+  B.fetch_rows(BK, klen);
   for (int kt = 0; kt < nk; ++kt) {
     char* cur = lds + (kt & 1) * STAGE;
     const unsigned nxt = lds_u + ((kt + 1) & 1) * STAGE;
@@ -323,9 +388,17 @@ __device__ __forceinline__ void mainloop(const AOp& A, const BOp& B, int klen, c
       A.zero_tail(cur, kt * BK, klen);
       B.zero_tail(cur + AOp::LDS_BYTES, kt * BK, klen);
     }
+    A.stage_rows(kt + 1);
+    B.stage_rows(kt + 1);
     __syncthreads();                 // ... everyone's have, and everyone is done reading `nxt`
+    A.take_rows(kt + 1);
+    B.take_rows(kt + 1);
     if (kt + 1 < nfull) issue_slice(A, B, nxt, (kt + 1) * BK);
     else if (tail && kt + 1 == nfull) issue_slice_tail(A, B, nxt, (kt + 1) * BK, klen);
+    if (kt + 2 < nk) {
+      A.fetch_rows((kt + 2) * BK, klen);
+      B.fetch_rows((kt + 2) * BK, klen);
+    }
     const char* ta = cur;
     const char* tb = cur + AOp::LDS_BYTES;
     i32x4 fa[2][TL::FM], fb[2][TL::FN];
@@ -1167,15 +1240,20 @@ struct XtYPlan {
   const int64_t* off;
   int E;
   int db_from_p;                          // 1: dY is P (row sums of the tile), 0: dY is Q
+  // X given as the token matrix it would be gathered from (row r of X = token row idx[r] / fan_out): the operand
+  // that holds X (Q when db_from_p, else P) reads its rows through idx; NULL: X is already in grouped order
+  const int64_t* idx;
+  int fan_out;
 };
 
-template <typename T, class TL>
+template <typename T, class TL, bool GA, bool GB>
 __global__ __launch_bounds__(TL::NT) void xty_mfma_kernel(XtYPlan a, Raster rast, int p_tiles) {
-  typedef TransOp<TL::BM, TL::NT> AOp;
-  typedef TransOp<TL::BN, TL::NT> BOp;
+  typedef TransOp<TL::BM, TL::NT, false, GA> AOp;
+  typedef TransOp<TL::BN, TL::NT, false, GB> BOp;
   constexpr int STAGE = AOp::LDS_BYTES + BOp::LDS_BYTES;
   __shared__ __attribute__((aligned(16))) char lds[2 * STAGE];
   __shared__ int64_t sDst[TL::BM];
+  __shared__ unsigned sRows[2 * 64];       // row offsets of a gathered operand (see TransOp)
 
   int m_tile, n_tile, m_loc, n_loc;
   if (!rast.map(blockIdx.x, m_tile, n_tile, m_loc, n_loc)) return;
@@ -1190,9 +1268,11 @@ __global__ __launch_bounds__(TL::NT) void xty_mfma_kernel(XtYPlan a, Raster rast
   __syncthreads();
 
   AOp A;
-  A.init((const char*)a.P + ((int64_t)r_lo * a.ldp + p0) * 2, a.ldp * 2, a.np - p0);
+  if constexpr (GA) A.init_gather((const char*)a.P + (int64_t)p0 * 2, a.ldp * 2, a.np - p0, a.idx + r_lo, a.fan_out, r_hi - r_lo, sRows);
+  else A.init((const char*)a.P + ((int64_t)r_lo * a.ldp + p0) * 2, a.ldp * 2, a.np - p0);
   BOp B;           // (rotated load order measured 1.5 % slower here, so both operands keep rot = 0)
-  B.init((const char*)a.Q + ((int64_t)r_lo * a.ldq + q0) * 2, a.ldq * 2, a.nq - q0);
+  if constexpr (GB) B.init_gather((const char*)a.Q + (int64_t)q0 * 2, a.ldq * 2, a.nq - q0, a.idx + r_lo, a.fan_out, r_hi - r_lo, sRows);
+  else B.init((const char*)a.Q + ((int64_t)r_lo * a.ldq + q0) * 2, a.ldq * 2, a.nq - q0);
 
   f32x16 acc[TL::FM][TL::FN];
   float rs[TL::FM];
@@ -1276,12 +1356,15 @@ static int launch_xty(const XtYArgs& a, hipStream_t st) {
   p.Db = a.Db; p.sdbe = a.sdbe; p.sdbn = a.sdbn;
   p.off = a.off; p.E = a.E;
   p.db_from_p = k_contig ? 1 : 0;
+  p.idx = a.idx; p.fan_out = a.fan_out;
   const int p_tiles = (p.np + TL::BM - 1) / TL::BM;
   const int q_tiles = (p.nq + TL::BN - 1) / TL::BN;
   const Raster r = make_raster((int64_t)a.E * p_tiles, q_tiles, GM_XTY);
   const int64_t grid = r.grid();
   if (grid > 0x7fffffffLL) { set_error("smoe_groupXtY: grid too large"); return SMOE_ERR_RANGE; }
-  hipLaunchKernelGGL((xty_mfma_kernel<T, TL>), dim3((unsigned)grid), dim3(TL::NT), 0, st, p, r, p_tiles);
+  if (a.idx == nullptr) hipLaunchKernelGGL((xty_mfma_kernel<T, TL, false, false>), dim3((unsigned)grid), dim3(TL::NT), 0, st, p, r, p_tiles);
+  else if (k_contig) hipLaunchKernelGGL((xty_mfma_kernel<T, TL, false, true>), dim3((unsigned)grid), dim3(TL::NT), 0, st, p, r, p_tiles);
+  else hipLaunchKernelGGL((xty_mfma_kernel<T, TL, true, false>), dim3((unsigned)grid), dim3(TL::NT), 0, st, p, r, p_tiles);
   int rc = launch_status("xty_mfma_kernel");
   if (rc == 0 && a.Db != nullptr && !k_contig) {
     hipLaunchKernelGGL(colsum_kernel<T>, dim3((a.N + 255) / 256, a.E), dim3(256), 0, st, (const T*)a.DY,
@@ -1299,6 +1382,13 @@ bool try_xty_mfma(const XtYArgs& a, int dtype, hipStream_t st, int& rc) {
   if (!aligned16(a.DY) || !aligned16(a.X)) return false;
   if (a.sdwk != 1 && a.sdwn != 1) return false;
   if (!fits_u32(BK * a.sdym * 2 + (int64_t)a.N * 2) || !fits_u32(BK * a.sxm * 2 + (int64_t)a.K * 2)) return false;
+  // gathered X: lane offsets are 32-bit byte offsets from the start of the token matrix
+  if (a.idx != nullptr && !fits_u32(((int64_t)a.L / a.fan_out) * a.sxm * 2 + (int64_t)a.K * 2)) return false;
+  // Looking the rows up costs the kernel about 4 % of its time; the gathered copy it saves costs 4 K bytes of HBM
+  // traffic per row against 2 K N flops, i.e. a share of the kernel time that shrinks with N.  Measured per training
+  // step: N = 1536 (Qwen-like, top-8) 9.12 -> 8.90 ms, N = 5760 (gpt-oss-like) 6.07 -> 6.03 ms, N = 28672 (Mixtral)
+  // 31.3 -> 31.5 ms: wide layers keep the separate pass.
+  if (a.idx != nullptr && a.N > XTY_GATHER_MAX_N) return false;
   rc = dtype == SMOE_BF16 ? launch_xty<bf16_t>(a, st) : launch_xty<f16_t>(a, st);
   return true;
 }

@@ -89,6 +89,24 @@ class HipBackend:
                 _C.stream_ptr(DY.device))
         _C.check(rc, "smoe_groupXtY")
 
+    @staticmethod
+    def xty_gathered(DY, X, idx, fan_out, DW, Db, off, E):
+        """groupXtY with X read through idx; False when the library has no such kernel for this call."""
+        _C.require_gpu(DY, "group_bwd_W")
+        lib = _C.load()
+        sdbe, sdbn = (Db.stride(0), Db.stride(1)) if Db is not None else (0, 0)
+        with _C.on_device(DY.device):
+            rc = lib.smoe_groupXtY_gathered(
+                _C.ptr(DY), DY.stride(0), DY.stride(1),
+                _C.ptr(X), X.stride(0), X.stride(1), _C.ptr(idx), fan_out,
+                _C.ptr(DW), DW.stride(0), DW.stride(1), DW.stride(2),
+                _C.ptr(Db), sdbe, sdbn,
+                _C.ptr(off), DY.size(0), X.size(1), DY.size(1), E, _C.float_code(DY.dtype),
+                _C.stream_ptr(DY.device))
+        if rc == _C.ERR_UNSUPPORTED:
+            return False
+        _C.check(rc, "smoe_groupXtY_gathered")
+        return True
 
     @staticmethod
     def combine(Y, gates, out, k):
@@ -427,8 +445,12 @@ def scatter2scatter_compileable(
 # ------------------------------------------------------------------------------------------------
 # groupXtY
 # ------------------------------------------------------------------------------------------------
-def group_bwd_W(DY, X, expert_offsets, E, has_bias=False, like=None):
+def group_bwd_W(DY, X, expert_offsets, E, has_bias=False, like=None, gather=None):
     """Per-expert dW / db over expert-grouped rows (reference ops.py:191-199).
+
+    `gather=(sorted_scattered_idxs, fan_out)`: X is not the grouped (L, K) matrix but the (L / fan_out, K) matrix it
+    would be gathered from, i.e. the call stands for `group_bwd_W(DY, group(X, idxs, fan_out=fan_out), ...)`
+    (reference parallel_experts.py:95-107) without the gathered copy ever being written.
 
     The returned DW is (E, K, N).  By default it is a view of a contiguous (E, N, K) buffer, so that after autograd
     undoes the `weight.permute(0, 2, 1)` of ParallelExperts the parameter gradient is contiguous.  `like` (the
@@ -442,6 +464,16 @@ def group_bwd_W(DY, X, expert_offsets, E, has_bias=False, like=None):
     else:
         DW = torch.empty((E, N, K), device=DY.device, dtype=DY.dtype).permute(0, 2, 1)
     Db = torch.empty((E, N), device=DY.device, dtype=DY.dtype) if has_bias else None
+    if gather is not None:
+        idx, fan_out = gather
+        assert idx.size(0) == DY.size(0) and X.size(0) * fan_out == DY.size(0)
+        if (not torch.compiler.is_compiling() and DY.is_cuda and hasattr(_backend, "xty_gathered")
+                and DY.dtype in (torch.bfloat16, torch.float16)):
+            _same_dtype("group_bwd_W", DY, X, DW, Db)
+            if _backend.xty_gathered(DY, X, _as_i64(idx).contiguous(), fan_out, DW, Db,
+                                     _as_i64(expert_offsets).contiguous(), E):
+                return DW, Db
+        X = group(X, idx, fan_out=fan_out)
     if torch.compiler.is_compiling():
         groupXtY_compileable(E, DW, Db, DY, X, expert_offsets)
     else:

@@ -71,13 +71,14 @@ class _GatedMLP(torch.autograd.Function):
         if need_x or need_w1 or need_b1:
             dpre = ops.scatter2scatter_glu_bwd(dy, w2.permute(0, 2, 1), pre, eid, idx, act=act, expert_offsets=off,
                                                alpha=ctx.alpha, limit=ctx.limit)
-            xg = ops.group(x, idx, fan_out=k)
             if need_w1 or need_b1:
-                d_w1, d_b1 = ops.group_bwd_W(DY=dpre, X=xg, expert_offsets=off, E=E, has_bias=b1 is not None, like=w1)
+                # the weight gradient reads the rows of x through idx: no gathered copy of x is made
+                d_w1, d_b1 = ops.group_bwd_W(DY=dpre, X=x, expert_offsets=off, E=E, has_bias=b1 is not None, like=w1,
+                                             gather=(idx, k))
                 d_w1 = d_w1 if need_w1 else None
             if need_x:
                 d_exp = ops.scatter2scatter(dpre, w1.permute(0, 2, 1), eid, idx, 1, x_grouped=True, y_grouped=False,
-                                            out=xg, expert_offsets=off)
+                                            expert_offsets=off)
                 d_x = ops.slot_sum(d_exp, x.size(0), k)
         return d_x, d_w1, (d_b1 if need_b1 else None), d_w2, (d_b2 if need_b2 else None), d_gates, \
             None, None, None, None, None, None, None

@@ -93,22 +93,20 @@ class ParallelLinear(torch.autograd.Function):
             dy = ops.group(grad_out, idx, coeff=coeff, fan_out=coeff_fan, out=dy_buf)
 
         d_w = d_b = None
-        xg = None
-        if need_w or need_b or (need_x and not grouped_in):
-            xg = x if grouped_in else ops.group(x, idx, fan_out=k)
         if need_w or need_b:
-            d_w, d_b = ops.group_bwd_W(DY=dy, X=xg, expert_offsets=off, E=E, has_bias=bias is not None, like=W)
+            # ungrouped input: the weight gradient reads the rows of x through idx (the reference gathers a copy
+            # of x first, parallel_experts.py:95-99)
+            d_w, d_b = ops.group_bwd_W(DY=dy, X=x, expert_offsets=off, E=E, has_bias=bias is not None, like=W,
+                                       gather=None if grouped_in else (idx, k))
             if not need_w:
                 d_w = None
 
         d_x = None
         if need_x:
-            # dX rows: dY @ W[e]^T, written grouped (grouped_in) or scattered back to slot order;
-            # the gathered copy of x is dead by now and is reused as the output buffer
+            # dX rows: dY @ W[e]^T, written grouped (grouped_in) or scattered back to slot order
             d_exp = ops.scatter2scatter(
                 X=dy, W=W.permute(0, 2, 1), k=1, x_grouped=True, y_grouped=grouped_in,
-                sorted_expert_idxs=eid, sorted_scattered_idxs=idx,
-                out=None if grouped_in else xg, expert_offsets=off)
+                sorted_expert_idxs=eid, sorted_scattered_idxs=idx, expert_offsets=off)
             d_x = ops.slot_sum(d_exp, x.size(0), k)
 
         return d_x, d_w, None, None, None, None, d_b, d_gates, None, None

@@ -192,3 +192,31 @@ def test_xty(T, E, k, K, N, out_layout, dtype):
     _close(Db, Db_ref, scale=0.1 * rows ** 0.5)
     for e in (torch.diff(off, prepend=torch.zeros(1, dtype=torch.long)) == 0).nonzero().flatten().tolist():
         assert not DW[e].any() and not Db[e].any()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("out_layout", ["param", "plain"])
+@pytest.mark.parametrize("T,E,k,K,N", [(4096, 8, 2, 512, 256), (1100, 8, 2, 200, 264), (130, 8, 3, 448, 72),
+                                       (2048, 32, 4, 192, 328), (700, 4, 1, 1024, 520), (3, 4, 2, 64, 64)])
+def test_xty_reads_tokens_through_the_index(T, E, k, K, N, out_layout, dtype):
+    """`group_bwd_W(..., gather=(idx, k))` - the weight gradient that picks the rows of the token matrix itself -
+    gives the bits of `group_bwd_W(DY, group(X, idx, fan_out=k), ...)`, the pair of the reference
+    (parallel_experts.py:95-107), in both output layouts, with bias gradient, ragged and empty experts; float32
+    (no gathering kernel) takes the grouped copy by itself.  And both agree with the oracle."""
+    experts, (eid, idx, off) = _routing(T, E, k, seed=N + 1, skew=2.0 if E == 32 else 0.0, empty=(1,) if E == 32 else ())
+    g = torch.Generator().manual_seed(K + 1)
+    X = torch.randn(T, K, generator=g).to(dtype)
+    DY = (torch.randn(T * k, N, generator=g) * 0.1).to(dtype)
+    like = None if out_layout == "param" else torch.empty(E, K, N, dtype=dtype, device=DEV)
+    Xd, DYd, idxd, offd = X.to(DEV), DY.to(DEV), idx.to(DEV), off.to(DEV)
+    DW, Db = ops.group_bwd_W(DYd, Xd, offd, E, has_bias=True, like=like, gather=(idxd, k))
+    DW2, Db2 = ops.group_bwd_W(DYd, ops.group(Xd, idxd, fan_out=k), offd, E, has_bias=True, like=like)
+    assert DW.stride() == DW2.stride()
+    assert torch.equal(DW, DW2) and torch.equal(Db, Db2)
+    DW_ref, Db_ref = oracle.group_bwd_W_ref(DY.float(), oracle.group_ref(X, idx, None, k).float(), off, E, has_bias=True)
+    rows = torch.diff(off, prepend=torch.zeros(1, dtype=torch.long)).max().item()
+    if dtype is not torch.float32:
+        _close(DW, DW_ref, scale=0.1 * rows ** 0.5)
+        _close(Db, Db_ref, scale=0.1 * rows ** 0.5)
+    else:
+        torch.testing.assert_close(DW.cpu(), DW_ref, rtol=1e-4, atol=1e-4)
