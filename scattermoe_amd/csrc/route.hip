@@ -3,7 +3,7 @@
 // torch.sort + bincount + cumsum.  Keys are tiny (expert ids), so a counting sort with an LDS
 // histogram per block and a wavefront match/rank scatter replaces the generic 64-bit radix sort.
 //
-// Small inputs (one chunk) run in ONE launch; larger ones in three:
+// Inputs of up to 16384 rows (one workgroup of 4 or 16 waves) run in ONE launch; larger ones in three:
 //   hist    : per-chunk LDS histogram                       -> counts[chunk][E]
 //   scan    : exclusive scan over (expert-major, chunk)     -> bases[chunk][E], off[E]
 //   scatter : stable rank inside the chunk + base           -> eid_out, idx_out
@@ -17,6 +17,9 @@ static constexpr int kRouteThreads = 256;
 static constexpr int kRouteWaves = kRouteThreads / 64;
 static constexpr int kRouteChunk = 4096;       // elements per block
 static constexpr int kRouteMaxE = 2048;        // LDS: (waves+1) * E ints
+static constexpr int kRouteFusedMax = 16384;   // rows one workgroup of 1024 threads sorts by itself (32768 rows take it
+                                               // 33 us, the three launches 28 us) ...
+static constexpr int kRouteFusedMaxE = 512;    // ... for at most this many experts (17 * E ints of LDS)
 
 template <typename I>
 __device__ __forceinline__ int load_id(const I* p, int64_t i) { return (int)p[i]; }
@@ -79,10 +82,11 @@ __device__ __forceinline__ void wave_scatter(const I* __restrict__ ids, int64_t 
 }
 
 // ---- single-launch path: whole input in one block ------------------------------------------------
-template <typename I>
-__global__ __launch_bounds__(kRouteThreads) void route_fused_kernel(
+template <typename I, int THREADS>
+__global__ __launch_bounds__(THREADS) void route_fused_kernel(
     const I* __restrict__ ids, int L, int E, int64_t* __restrict__ eid_out,
     int64_t* __restrict__ idx_out, int64_t* __restrict__ off_out) {
+  constexpr int kRouteThreads = THREADS, kRouteWaves = THREADS / 64;      // this kernel's own block shape
   extern __shared__ int lds[];          // [kRouteWaves][E] wave histograms/bases, then [E] totals
   int* hist = lds;
   int* total = lds + kRouteWaves * E;
@@ -148,23 +152,31 @@ __global__ __launch_bounds__(kRouteThreads) void route_hist_kernel(
   for (int i = tid; i < E; i += kRouteThreads) counts[(int64_t)blockIdx.x * E + i] = lds[i];
 }
 
-// One block.  counts[c][e] -> exclusive position of chunk c's first row of expert e.
+// One block of 16 waves.  counts[c][e] -> exclusive position of chunk c's first row of expert e.
+// A wave takes the experts e = wave, wave + 16, ...; its lanes take 64 chunks at a time (wave-wide scan, carry
+// between the groups of 64), so the walk over the chunks of an expert is 64 wide instead of serial.
 __global__ __launch_bounds__(1024) void route_scan_kernel(int* __restrict__ counts, int nchunk, int E,
                                                          int64_t* __restrict__ off_out) {
   extern __shared__ int total[];  // [E]
-  const int tid = threadIdx.x;
-  for (int e = tid; e < E; e += blockDim.x) {
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  for (int e = w; e < E; e += 16) {
     int run = 0;
-    for (int c = 0; c < nchunk; ++c) {
-      const int v = counts[(int64_t)c * E + e];
-      counts[(int64_t)c * E + e] = run;
-      run += v;
+    for (int c0 = 0; c0 < nchunk; c0 += 64) {
+      const int c = c0 + lane;
+      const int v = c < nchunk ? counts[(int64_t)c * E + e] : 0;
+      int incl = v;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        int u = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += u;
+      }
+      if (c < nchunk) counts[(int64_t)c * E + e] = run + incl - v;
+      run += __shfl(incl, 63, 64);
     }
-    total[e] = run;
+    if (lane == 0) total[e] = run;
   }
   __syncthreads();
   if (tid < 64) {
-    const int lane = tid;
     int carry = 0;
     for (int e0 = 0; e0 < E; e0 += 64) {
       const int e = e0 + lane;
@@ -212,7 +224,7 @@ __global__ __launch_bounds__(kRouteThreads) void route_scatter_kernel(
 }
 
 size_t route_workspace_bytes(int64_t L, int E) {
-  if (L <= kRouteChunk) return 0;
+  if (L <= kRouteChunk || (L <= kRouteFusedMax && E <= kRouteFusedMaxE)) return 0;
   return (size_t)cdiv64(L, kRouteChunk) * (size_t)E * sizeof(int);
 }
 
@@ -221,7 +233,14 @@ static int launch_route_t(const I* ids, int64_t L, int E, int64_t* eid_out, int6
                           int64_t* off_out, void* ws, hipStream_t st) {
   if (L <= kRouteChunk) {
     const size_t lds = (size_t)(kRouteWaves + 1) * E * sizeof(int);
-    hipLaunchKernelGGL(route_fused_kernel<I>, dim3(1), dim3(kRouteThreads), lds, st, ids, (int)L, E,
+    hipLaunchKernelGGL((route_fused_kernel<I, kRouteThreads>), dim3(1), dim3(kRouteThreads), lds, st, ids, (int)L, E,
+                       eid_out, idx_out, off_out);
+    return launch_status("route_fused_kernel");
+  }
+  if (L <= kRouteFusedMax && E <= kRouteFusedMaxE) {
+    // one workgroup of 16 waves: a launch costs more than sorting 2048 rows per wave does
+    const size_t lds = (size_t)(1024 / 64 + 1) * E * sizeof(int);
+    hipLaunchKernelGGL((route_fused_kernel<I, 1024>), dim3(1), dim3(1024), lds, st, ids, (int)L, E,
                        eid_out, idx_out, off_out);
     return launch_status("route_fused_kernel");
   }

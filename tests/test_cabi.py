@@ -30,11 +30,13 @@ def test_library_exports_declared_symbols():
 def test_argument_errors_need_no_gpu():
     lib = C.load()
     assert lib.smoe_route_workspace_bytes(4096, 8) == 0
-    assert lib.smoe_route_workspace_bytes(4097, 8) == 2 * 8 * 4
+    assert lib.smoe_route_workspace_bytes(16384, 512) == 0          # one workgroup sorts up to 16384 rows by itself
+    assert lib.smoe_route_workspace_bytes(16385, 8) == 5 * 8 * 4
+    assert lib.smoe_route_workspace_bytes(4097, 513) == 2 * 513 * 4
     assert lib.smoe_route(None, 0, 16, 8, None, None, None, None, 0, None) == -1          # SMOE_ERR_NULL
     assert b"NULL" in lib.smoe_last_error()
     assert lib.smoe_route(None, 0, -1, 8, None, None, None, None, 0, None) == -2          # SMOE_ERR_SHAPE
     assert lib.smoe_group(None, 0, 0, None, None, 0, 0, None, 4, 4, 1, 9, None) == -3       # SMOE_ERR_DTYPE
     one = ctypes.c_void_p(16)
-    assert lib.smoe_route(one, 0, 10000, 8, one, one, one, None, 0, None) == -4           # SMOE_ERR_WORKSPACE
+    assert lib.smoe_route(one, 0, 100000, 8, one, one, one, None, 0, None) == -4          # SMOE_ERR_WORKSPACE
     assert lib.smoe_route(one, 0, 1 << 33, 8, one, one, one, one, 1 << 40, None) == -5    # SMOE_ERR_RANGE

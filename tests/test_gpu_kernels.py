@@ -35,7 +35,8 @@ def _experts(T, E, k, seed, skew=False):
 # routing: bit-exact
 # ---------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("T,E,k", [(1, 8, 2), (3, 1, 1), (256, 8, 2), (512, 8, 4), (2048, 8, 2), (2049, 8, 2),
-                                   (8192, 32, 4), (32768, 128, 8), (16384, 8, 2), (5000, 300, 3), (70000, 64, 1)])
+                                   (8192, 32, 4), (32768, 128, 8), (16384, 8, 2), (5000, 300, 3), (70000, 64, 1),
+                                   (4096, 512, 8), (2000, 700, 5), (16385, 8, 2), (40000, 2000, 1)])
 @pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
 def test_route_bit_exact(T, E, k, dtype):
     experts = _experts(T, E, k, seed=T + E, skew=(E >= 32)).to(dtype)

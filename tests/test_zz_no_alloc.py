@@ -42,8 +42,9 @@ def test_route_static_matches_route_on_two_calls_in_a_row():
     with torch.cuda.device(0):
         assert lib.smoe_route_static_init() == 0, lib.smoe_last_error()
         # large first (64 chunks x 128 experts of histograms), then smaller inputs that reuse the same buffer
-        for L, E, dtype in [(262144, 128, torch.int64), (32768, 8, torch.int64), (10001, 33, torch.int32),
-                            (4097, 5, torch.int64), (300, 8, torch.int64)]:
+        # (the last three are sorted by one workgroup, without the buffer)
+        for L, E, dtype in [(262144, 128, torch.int64), (100000, 600, torch.int64), (40000, 33, torch.int32),
+                            (32768, 8, torch.int64), (4097, 5, torch.int64), (300, 8, torch.int64)]:
             ids = _ids(L, E, seed=L + E).to(dtype)
             got = _route(lib, "static", ids.to(DEV), E)
             want = _route(lib, "workspace", ids.to(DEV), E)
