@@ -133,6 +133,12 @@ class TimedBackend:
         return self._timed(lambda: self.inner.xty(DY, X, DW, Db, off, E) is None,
                            2.0 * DY.size(0) * X.size(1) * DY.size(1), None, name)
 
+    def xty_gathered(self, DY, X, idx, fan_out, DW, Db, off, E):
+        # only the layer-1 weight gradient reads its X operand through the index vector; a declined launch
+        # (False) is not recorded: the caller then runs group + xty, and that launch is
+        return self._timed(lambda: self.inner.xty_gathered(DY, X, idx, fan_out, DW, Db, off, E),
+                           2.0 * DY.size(0) * X.size(1) * DY.size(1), None, "l1_dw")
+
     def _timed(self, fn, flops, k_contig, name):
         if not self.on:
             return fn()
