@@ -2,7 +2,8 @@
 //
 // One workgroup owns one BM x BN output tile that never straddles two experts and walks the contraction in
 // slices of 64: global -> LDS directly (double buffered, or a ring of stages for the memory-bound small-row
-// classes) -> MFMA 32x32x16 -> LDS-staged epilogue with 16-byte global accesses.
+// classes), or global -> registers -> LDS in the one-wave-per-SIMD form of the 256 x 256 class (mainloop_rs)
+// -> MFMA 32x32x16 -> LDS-staged epilogue with 16-byte global accesses.
 // Operands whose contraction axis is contiguous in memory ("direct": gathered X rows, weights stored
 // (N,K)) sit in LDS as [row][64] with a 16-byte XOR swizzle and are read with ds_read_b128; operands
 // whose contraction axis is strided ("transposed": weights stored (K,N), both operands of X^T dY) sit
@@ -153,6 +154,12 @@ struct DirectOp {
   __device__ __forceinline__ void issue_one(unsigned tile, int k0, int j) const {
     load_to_lds16<STREAM>(base + (int64_t)k0 * 2, off[j], tile + wave_uniform_id() * 1024 + rnd(j) * NT * 16);
   }
+  // the same piece into registers, and where it belongs in the LDS tile
+  __device__ __forceinline__ i32x4 load_piece(int k0, int j) const {
+    const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)(base + (int64_t)k0 * 2), 0, -1, 0x00020000);
+    return __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)off[j], 0, 0));
+  }
+  __device__ __forceinline__ int piece_lds(int j) const { return (rnd(j) * NT + (int)threadIdx.x) * 16; }
   __device__ __forceinline__ void issue(unsigned tile, int k0) const {
 #pragma unroll
     for (int j = 0; j < R; ++j) issue_one(tile, k0, j);
@@ -285,6 +292,12 @@ struct TransOp {
     if constexpr (GATHER) load_to_lds16<STREAM>(make_uniform(base), off[j], tile + wave_uniform_id() * 1024 + rnd(j) * NT * 16);
     else load_to_lds16<STREAM>(base + (int64_t)k0 * ld, off[j], tile + wave_uniform_id() * 1024 + rnd(j) * NT * 16);
   }
+  // the same piece into registers (not for gathered rows), and where it belongs in the LDS tile
+  __device__ __forceinline__ i32x4 load_piece(int k0, int j) const {
+    const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)(base + (int64_t)k0 * ld), 0, -1, 0x00020000);
+    return __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)off[j], 0, 0));
+  }
+  __device__ __forceinline__ int piece_lds(int j) const { return (rnd(j) * NT + (int)threadIdx.x) * 16; }
   __device__ __forceinline__ void issue(unsigned tile, int k0) const {
 #pragma unroll
     for (int j = 0; j < R; ++j) issue_one(tile, k0, j);
@@ -351,10 +364,11 @@ __device__ __forceinline__ void issue_slice_tail(const AOp& A, const BOp& B, uns
   }
 }
 
-template <int BM_, int BN_, int WM_, int WN_, int NS_ = 2>
+template <int BM_, int BN_, int WM_, int WN_, int NS_ = 2, bool RS_ = false>
 struct Tile {
   static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_;
   static constexpr int NS = NS_;                      // LDS stages (2: double buffer, more: ring)
+  static constexpr bool RS = RS_;                     // operands travel global -> registers -> LDS (mainloop_rs)
   static constexpr int NW = WM * WN, NT = NW * 64;
   static constexpr int WTM = BM / WM, WTN = BN / WN;
   static constexpr int FM = WTM / 32, FN = WTN / 32;
@@ -440,6 +454,110 @@ __device__ __forceinline__ void mainloop(AOp& A, BOp& B, int klen, char* lds, bo
       __builtin_amdgcn_sched_barrier(0);
     }
   }
+}
+
+// Main loop of the one-wave-per-SIMD class (4 waves, 128 x 128 wave tiles): operands travel global -> registers ->
+// LDS.  A burst of loads at the top of a slice holds the waves that issue it off the matrix pipe until the memory
+// pipeline has taken all of them (it takes one 1 KB wave-load per ~17 cycles and CU), and loads spread over the
+// slice leave the late ones too little time to land when LDS is the only place they can land in: here every
+// thread's 16 pieces of a slice sit in registers for up to two slices, which LDS has no room for.
+//   set S = (kt + 1) & 1 holds slice kt + 1: its pieces are written to the other LDS stage during steps 0-2 of
+//   slice kt (ds_write_b128, second half of each step) and each is reloaded with slice kt + 3 one step later
+//   (pieces 12-15 in step 0 of the next slice), one load per 4 MFMAs throughout;
+//   one barrier per slice, after step 2: behind it the fragments of step 0 of slice kt + 1 are read while the
+//   MFMAs of step 3 run.
+// Whole 64-deep slices only, at least two of them (the launcher checks); loads past the end re-read the last slice.
+template <typename T, class TL, class AOp, class BOp, int P>
+__device__ __forceinline__ void rs_slice(const AOp& A, const BOp& B, char* lds, int kt, int last_k0, int wm, int wn,
+                                         f32x16 (&acc)[TL::FM][TL::FN], i32x4 (&g)[2][16],
+                                         i32x4 (&fa)[2][TL::FM], i32x4 (&fb)[2][TL::FN]) {
+  constexpr int STAGE = AOp::LDS_BYTES + BOp::LDS_BYTES;
+  constexpr int FM = TL::FM, FN = TL::FN, NM = FM * FN;
+  constexpr int DR = FM * AOp::DS_PER_FRAG + FN * BOp::DS_PER_FRAG;      // fragment reads per step
+  static_assert(NM == 16 && DR >= 8 && DR <= 16, "pipeline below is laid out for 16 MFMAs per step");
+  char* cur = lds + P * STAGE;
+  char* nxt = lds + (P ^ 1) * STAGE;
+  constexpr int S = P ^ 1;
+  const int k2 = min((kt + 2) * BK, last_k0), k3 = min((kt + 3) * BK, last_k0);
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) {
+    const int c = ks & 1, n = c ^ 1;
+    const char* src = ks < 3 ? cur : nxt;
+    const int step = ks < 3 ? ks + 1 : 0;
+#pragma unroll
+    for (int i = 0; i < FM; ++i) fa[n][i] = AOp::frag(src, wm * TL::WTM + i * 32, step);
+#pragma unroll
+    for (int j = 0; j < FN; ++j) fb[n][j] = BOp::frag(src + AOp::LDS_BYTES, wn * TL::WTN + j * 32, step);
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int j = 0; j < FN; ++j) acc[i][j] = Mfma<T>::run(fb[c][j], fa[c][i], acc[i][j]);
+    // pieces written in this step: 0-5, 6-10, 11-15, none
+    constexpr int W0[5] = {0, 6, 11, 16, 16};
+#pragma unroll
+    for (int q = W0[ks]; q < W0[ks + 1]; ++q) {
+      if (q & 1) lds_write16(nxt + AOp::LDS_BYTES + B.piece_lds(q >> 1), g[S][q]);
+      else lds_write16(nxt + A.piece_lds(q >> 1), g[S][q]);
+    }
+    // pieces loaded in this step: 12-15 of the other set (slice kt + 2), then 0-3, 4-7, 8-11 of this one (slice kt + 3)
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int q = ks == 0 ? 12 + u : (ks - 1) * 4 + u;
+      const int k0 = ks == 0 ? k2 : k3;
+      i32x4& dst = ks == 0 ? g[P][q] : g[S][q];
+      dst = (q & 1) ? B.load_piece(k0, q >> 1) : A.load_piece(k0, q >> 1);
+    }
+#pragma unroll
+    for (int m = 0; m < NM; ++m) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if (m < DR - 8) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      else if (m < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      else if (m - 8 < W0[ks + 1] - W0[ks]) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+      if (m % 4 == 3) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (ks == 2) {
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // this thread's pieces are in LDS, its reads of `cur` done
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+}
+
+template <typename T, class TL, class AOp, class BOp>
+__device__ __forceinline__ void mainloop_rs(const AOp& A, const BOp& B, int klen, char* lds,
+                                            f32x16 (&acc)[TL::FM][TL::FN]) {
+  static_assert(AOp::R == 8 && BOp::R == 8 && BK == 64, "16 pieces per thread and slice");
+  const int wave = threadIdx.x >> 6;
+  const int wm = wave / TL::WN, wn = wave % TL::WN;
+  const int nk = klen / BK;
+  const int last_k0 = (nk - 1) * BK;
+  i32x4 g[2][16];
+  i32x4 fa[2][TL::FM], fb[2][TL::FN];
+#pragma unroll
+  for (int q = 0; q < 16; ++q) g[0][q] = (q & 1) ? B.load_piece(0, q >> 1) : A.load_piece(0, q >> 1);
+#pragma unroll
+  for (int q = 0; q < 16; ++q) g[1][q] = (q & 1) ? B.load_piece(min(BK, last_k0), q >> 1) : A.load_piece(min(BK, last_k0), q >> 1);
+#pragma unroll
+  for (int q = 0; q < 16; ++q) {
+    if (q & 1) lds_write16(lds + AOp::LDS_BYTES + B.piece_lds(q >> 1), g[0][q]);
+    else lds_write16(lds + A.piece_lds(q >> 1), g[0][q]);
+  }
+#pragma unroll
+  for (int q = 0; q < 12; ++q) g[0][q] = (q & 1) ? B.load_piece(min(2 * BK, last_k0), q >> 1) : A.load_piece(min(2 * BK, last_k0), q >> 1);
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int i = 0; i < TL::FM; ++i) fa[0][i] = AOp::frag(lds, wm * TL::WTM + i * 32, 0);
+#pragma unroll
+  for (int j = 0; j < TL::FN; ++j) fb[0][j] = BOp::frag(lds + AOp::LDS_BYTES, wn * TL::WTN + j * 32, 0);
+  int kt = 0;
+  for (; kt + 1 < nk; kt += 2) {
+    rs_slice<T, TL, AOp, BOp, 0>(A, B, lds, kt, last_k0, wm, wn, acc, g, fa, fb);
+    rs_slice<T, TL, AOp, BOp, 1>(A, B, lds, kt + 1, last_k0, wm, wn, acc, g, fa, fb);
+  }
+  if (kt < nk) rs_slice<T, TL, AOp, BOp, 0>(A, B, lds, kt, last_k0, wm, wn, acc, g, fa, fb);
 }
 
 // Main loop of the small-row (decode) tile class: memory bound, so what matters is bytes in flight.  The
@@ -555,11 +673,17 @@ __device__ __forceinline__ int staged_addr(int row, int col) {
 
 // `bias_of(tile_col)` returns the value to add to that column (0 without bias).
 template <typename T, class TL, typename BF>
-__device__ __forceinline__ void stage_accumulators(const f32x16 (&acc)[TL::FM][TL::FN], char* lds, BF bias_of) {
+__device__ __forceinline__ void stage_accumulators(const f32x16 (&acc)[TL::FM][TL::FN], char* lds, BF bias_of,
+                                                   float* sbias) {
   typedef T T4 __attribute__((ext_vector_type(4)));
   static_assert(TL::BM * TL::BN * 2 <= TL::NS * (TL::BM + TL::BN) * 128, "staged tile must fit the operand buffers");
   const int wave = threadIdx.x >> 6, l = lane_id();
   const int wm = wave / TL::WN, wn = wave % TL::WN;
+  // One wave per SIMD: the additions per column come from LDS (written here, one column per thread), so that the
+  // walk over the 256 accumulator registers below is one straight piece of code without loads or branches.
+  if constexpr (TL::RS) {
+    for (int t = threadIdx.x; t < TL::BN; t += TL::NT) sbias[t] = bias_of(t);
+  }
   __syncthreads();                                   // every wave is done reading operands
 #pragma unroll
   for (int j = 0; j < TL::FN; ++j) {
@@ -567,8 +691,15 @@ __device__ __forceinline__ void stage_accumulators(const f32x16 (&acc)[TL::FM][T
     for (int g = 0; g < 4; ++g) {
       const int col = wn * TL::WTN + j * 32 + g * 8 + (l >> 5) * 4;
       float bv[4];
+      if constexpr (TL::RS) {
+        typedef float f32x4_t __attribute__((ext_vector_type(4)));
+        const f32x4_t b4 = *(const f32x4_t*)(sbias + col);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) bv[e] = bias_of(col + e);
+        for (int e = 0; e < 4; ++e) bv[e] = b4[e];
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) bv[e] = bias_of(col + e);
+      }
 #pragma unroll
       for (int i = 0; i < TL::FM; ++i) {
         const int row = wm * TL::WTM + i * 32 + (l & 31);
@@ -719,13 +850,13 @@ __device__ __forceinline__ void stream_store(const V& v, V* p) { __builtin_nonte
 template <typename T, class TL>
 __device__ __forceinline__ void epilogue_staged(const f32x16 (&acc)[TL::FM][TL::FN], T* __restrict__ out,
                                                 const int64_t* dst, int n0, int ncols, const T* __restrict__ bias,
-                                                int64_t sb, char* lds) {
+                                                int64_t sb, char* lds, float* sbias = nullptr) {
   typedef T T8 __attribute__((ext_vector_type(8)));
   constexpr int CPR = TL::BN / 8, PIECES = TL::BM * CPR, PP = PIECES / TL::NT;
   static_assert(PIECES % TL::NT == 0, "pieces must divide evenly");
   stage_accumulators<T, TL>(acc, lds, [&](int tc) {
     return bias != nullptr && n0 + tc < ncols ? to_f32(bias[(int64_t)(n0 + tc) * sb]) : 0.0f;
-  });
+  }, sbias);
 #pragma unroll
   for (int q = 0; q < PP; ++q) {
     const int p = q * TL::NT + threadIdx.x;
@@ -740,7 +871,7 @@ __device__ __forceinline__ void epilogue_staged(const f32x16 (&acc)[TL::FM][TL::
 template <typename T, class TL>
 __device__ __forceinline__ void epilogue_glu_fwd_staged(const f32x16 (&acc)[TL::FM][TL::FN], const S2SArgs& a,
                                                         int row0, int rows, int nh0, const T* __restrict__ bias,
-                                                        char* lds) {
+                                                        char* lds, float* sbias = nullptr) {
   {
     typedef T T8 __attribute__((ext_vector_type(8)));
     constexpr int HALF = TL::WTN / 2;
@@ -751,7 +882,7 @@ __device__ __forceinline__ void epilogue_glu_fwd_staged(const f32x16 (&acc)[TL::
       const int j = tc % TL::WTN;
       const int hc = nh0 + (tc / TL::WTN) * HALF + j % HALF;
       return bias != nullptr && hc < F ? to_f32(bias[(int64_t)(hc + (j >= HALF ? F : 0)) * a.sbn]) : 0.0f;
-    });
+    }, sbias);
     const bool gf = (a.act & 1) != 0;
     T* pre = (T*)a.Y;
     T* hid = (T*)a.H;
@@ -782,11 +913,11 @@ __device__ __forceinline__ void epilogue_glu_fwd_staged(const f32x16 (&acc)[TL::
 // two coalesced 16-byte loads of the saved pre-activation, two coalesced 16-byte stores of its gradient.
 template <typename T, class TL>
 __device__ __forceinline__ void epilogue_glu_bwd_staged(const f32x16 (&acc)[TL::FM][TL::FN], const S2SArgs& a,
-                                                        int row0, int rows, int n0, char* lds) {
+                                                        int row0, int rows, int n0, char* lds, float* sbias = nullptr) {
   typedef T T8 __attribute__((ext_vector_type(8)));
   constexpr int CPR = TL::BN / 8, PIECES = TL::BM * CPR, PP = PIECES / TL::NT, GRP = PP < 4 ? PP : 4;
   static_assert(PIECES % TL::NT == 0 && PP % GRP == 0, "pieces must divide evenly");
-  stage_accumulators<T, TL>(acc, lds, [](int) { return 0.0f; });
+  stage_accumulators<T, TL>(acc, lds, [](int) { return 0.0f; }, sbias);
   const int F = a.N;
   const bool gf = (a.act & 1) != 0;
   const T* pre = (const T*)a.aux;
@@ -836,14 +967,14 @@ __device__ __forceinline__ void epilogue_glu_bwd_staged(const f32x16 (&acc)[TL::
 template <typename T, class TL>
 __device__ __forceinline__ void epilogue_oss_fwd_staged(const f32x16 (&acc)[TL::FM][TL::FN], const S2SArgs& a,
                                                         int row0, int rows, int n0, const T* __restrict__ bias,
-                                                        char* lds) {
+                                                        char* lds, float* sbias = nullptr) {
   typedef T T8 __attribute__((ext_vector_type(8)));
   typedef T T4 __attribute__((ext_vector_type(4)));
   constexpr int CPR = TL::BN / 8, PIECES = TL::BM * CPR, PP = PIECES / TL::NT;
   static_assert(PIECES % TL::NT == 0, "pieces must divide evenly");
   stage_accumulators<T, TL>(acc, lds, [&](int tc) {
     return bias != nullptr && n0 + tc < a.N ? to_f32(bias[(int64_t)(n0 + tc) * a.sbn]) : 0.0f;
-  });
+  }, sbias);
   T* pre = (T*)a.Y;
   T* hid = (T*)a.H;
 #pragma unroll
@@ -865,11 +996,11 @@ __device__ __forceinline__ void epilogue_oss_fwd_staged(const f32x16 (&acc)[TL::
 // pre-activation pairs and two 16-byte stores of their gradient.
 template <typename T, class TL>
 __device__ __forceinline__ void epilogue_oss_bwd_staged(const f32x16 (&acc)[TL::FM][TL::FN], const S2SArgs& a,
-                                                        int row0, int rows, int n0, char* lds) {
+                                                        int row0, int rows, int n0, char* lds, float* sbias = nullptr) {
   typedef T T8 __attribute__((ext_vector_type(8)));
   constexpr int CPR = TL::BN / 8, PIECES = TL::BM * CPR, PP = PIECES / TL::NT, GRP = PP < 4 ? PP : 4;
   static_assert(PIECES % TL::NT == 0 && PP % GRP == 0, "pieces must divide evenly");
-  stage_accumulators<T, TL>(acc, lds, [](int) { return 0.0f; });
+  stage_accumulators<T, TL>(acc, lds, [](int) { return 0.0f; }, sbias);
   const int F = a.N;
   const T* pre = (const T*)a.aux;
   T* dpre = (T*)a.Y;
@@ -1007,6 +1138,7 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
   __shared__ __attribute__((aligned(16))) char lds[TL::NS * STAGE];
   __shared__ int64_t sDst[TL::BM];
   __shared__ int sSrc[TL::BM];
+  __shared__ __attribute__((aligned(16))) float sBias[TL::RS ? TL::BN : 4];
 
   int m_tile, n_tile, m_loc, n_loc;
   if (!rast.map(blockIdx.x, m_tile, n_tile, m_loc, n_loc)) return;
@@ -1030,7 +1162,7 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
   __syncthreads();
 
   AOp A;
-  A.rot = (n_loc * AOp::R / Raster::SN) % AOp::R;      // the row panel has SN sharers
+  A.rot = TL::RS ? 0 : (n_loc * AOp::R / Raster::SN) % AOp::R;      // the row panel has SN sharers
   // Lane offsets are 32-bit: grouped input rows are taken relative to the tile's first row (so that the input may
   // be of any size), gathered ones relative to the start of the token matrix.
   const int64_t sxm = a.sxm;
@@ -1038,7 +1170,7 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
   const char* Xb = (const char*)a.X + (int64_t)src0 * sxm * 2;
   A.init(Xb, [&](int row) { return (int64_t)(sSrc[row] - src0) * sxm * 2; });
   BOp B;
-  B.rot = (m_loc * BOp::R / Raster::SM) % BOp::R;      // the column panel has SM sharers
+  B.rot = TL::RS ? 0 : (m_loc * BOp::R / Raster::SM) % BOp::R;      // the column panel has SM sharers
   const char* Wb = (const char*)a.W + (int64_t)e * a.swe * 2;
   if (a.glu == 1) {
     // tile column tc -> weight column: wave block tc / WTN, first half of the block from [0, F), second from [F, 2F)
@@ -1070,12 +1202,20 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
     for (int j = 0; j < TL::FN; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-  if constexpr (TL::NS > 2) mainloop_ring<T, TL, AOp, BOp>(A, B, a.K, lds, acc);
+  if constexpr (TL::RS) mainloop_rs<T, TL, AOp, BOp>(A, B, a.K, lds, acc);
+  else if constexpr (TL::NS > 2) mainloop_ring<T, TL, AOp, BOp>(A, B, a.K, lds, acc);
   else mainloop<T, TL, AOp, BOp, false>(A, B, a.K, lds, false, acc, rs);
 
   const T* bias = a.b ? (const T*)a.b + (int64_t)e * a.sbe : nullptr;
-  // 16-byte pieces need every row start 16-byte aligned; otherwise the lane-wise epilogues are used
-  if (a.glu == 0) {
+  // 16-byte pieces need every row start 16-byte aligned; otherwise the lane-wise epilogues are used (the
+  // one-wave-per-SIMD class is only launched on aligned outputs)
+  if constexpr (TL::RS) {
+    if (a.glu == 0) epilogue_staged<T, TL>(acc, (T*)a.Y, sDst, n0, a.N, bias, a.sbn, lds, sBias);
+    else if (a.glu == 1) epilogue_glu_fwd_staged<T, TL>(acc, a, row0, rows, n0, bias, lds, sBias);
+    else if (a.glu == 2) epilogue_glu_bwd_staged<T, TL>(acc, a, row0, rows, n0, lds, sBias);
+    else if (a.glu == 3) epilogue_oss_fwd_staged<T, TL>(acc, a, row0, rows, n0, bias, lds, sBias);
+    else epilogue_oss_bwd_staged<T, TL>(acc, a, row0, rows, n0, lds, sBias);
+  } else if (a.glu == 0) {
     const bool al16 = (((uintptr_t)a.Y & 15) == 0) && ((a.sym | a.N) & 7) == 0;
     if (al16) epilogue_staged<T, TL>(acc, (T*)a.Y, sDst, n0, a.N, bias, a.sbn, lds);
     else epilogue<T, TL>(acc, (T*)a.Y, sDst, n0, a.N, bias, a.sbn);
@@ -1163,6 +1303,23 @@ static int tail_split(const S2SArgs& a) {
   return (int)m_first;
 }
 
+// The 256 x 256 class.  Products with a long enough contraction run on the one-wave-per-SIMD form of it
+// (mainloop_rs: Mixtral shape, per 64-deep slice 2 420-2 550 cycles against 2 890-3 000; its prologue and its
+// epilogue, run by half as many threads, cost about 5 000 cycles more per tile, which a 12-slice contraction does not
+// earn back: K = 768 is 5 % slower, K = 1536 even, K = 2048 is 5-8 % faster).  The fused gated-unit gradient stays with
+// the 8-wave form: its epilogue is bound by vector-ALU work that 8 waves overlap better (Mixtral: 3.91 against 4.04 ms).
+// Both forms add up every output element in the same order: the same bits.
+static constexpr int RS_MIN_K = 1792;
+template <typename T>
+static int launch_main(const S2SArgs& a, bool b_tr, hipStream_t st) {
+  bool al16 = true;             // the one-wave-per-SIMD form has only the LDS-staged epilogues (16-byte pieces)
+  if (a.glu == 0) al16 = (((uintptr_t)a.Y & 15) == 0) && ((a.sym | a.N) & 7) == 0;
+  else if (a.glu == 1) al16 = ((((uintptr_t)a.Y | (uintptr_t)a.H) & 15) == 0) && ((a.sym | a.shm | a.N) & 7) == 0;
+  if (al16 && a.glu != 2 && a.glu != 4 && a.K % BK == 0 && a.K >= RS_MIN_K)
+    return launch_s2s<T, Tile<256, 256, 2, 2, 2, true>>(a, b_tr, st);
+  return launch_s2s<T, Tile<256, 256, 2, 4>>(a, b_tr, st);
+}
+
 template <typename T>
 static int dispatch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
   // the gpt-oss epilogues exist only in their LDS-staged form (16-byte pieces)
@@ -1177,17 +1334,17 @@ static int dispatch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
     first.m_count = m_first;
     rest.m_begin = m_first;
     // both classes have 256-row tiles, hence the same numbering of the tile rows
-    if (const int rc = launch_s2s<T, Tile<256, 256, 2, 4>>(first, b_tr, st)) return rc;
+    if (const int rc = launch_main<T>(first, b_tr, st)) return rc;
     return launch_s2s<T, Tile<256, 128, 4, 2, 3>>(rest, b_tr, st);
   }
-  if (avg >= ROWS256_BELOW && !half_width_wins(a)) return launch_s2s<T, Tile<256, 256, 2, 4>>(a, b_tr, st);
+  if (avg >= ROWS256_BELOW && !half_width_wins(a)) return launch_main<T>(a, b_tr, st);
   // Wide launches (enough 256-wide tile columns to fill the chip twice even with one tile row per expert, e.g.
   // Mixtral layer 1) move half as many token rows per weight byte with 256-wide tiles as with 128-wide ones:
   // the 256 x 256 class from 136 rows per expert on (544..832 Mixtral tokens: layer 1 -9..-11 % against the
   // 256 x 128 ring), 128 x 256 ring tiles below (experts of about one 128-row tile: 448 tokens 518 -> 373 us,
   // 512 tokens 520 -> 455 us).  Launches with few tile columns (Mixtral layer 2) are faster in the classes below.
   const bool wide = (int64_t)a.E * ((a.N + (a.glu == 1 ? 127 : 255)) / (a.glu == 1 ? 128 : 256)) >= 2 * NUM_CU;
-  if (wide && avg >= ROWS128W_BELOW) return launch_s2s<T, Tile<256, 256, 2, 4>>(a, b_tr, st);
+  if (wide && avg >= ROWS128W_BELOW) return launch_main<T>(a, b_tr, st);
   if (wide && avg >= ROWS64_BELOW) return launch_s2s<T, Tile<128, 256, 2, 4, 3>>(a, b_tr, st);
   // Below that the launch is a stream over the weights: ring-buffered classes, tile height by rows per expert
   if (avg >= ROWS128_BELOW) return launch_s2s<T, Tile<256, 128, 4, 2, 3>>(a, b_tr, st);
@@ -1398,3 +1555,4 @@ bool try_xty_mfma(const XtYArgs& a, int dtype, hipStream_t st, int& rc) {
 }
 
 }  // namespace smoe
+
