@@ -155,7 +155,8 @@ struct DirectOp {
     load_to_lds16<STREAM>(base + (int64_t)k0 * 2, off[j], tile + wave_uniform_id() * 1024 + rnd(j) * NT * 16);
   }
   // the same piece into registers, and where it belongs in the LDS tile
-  __device__ __forceinline__ i32x4 load_piece(int k0, int j) const {
+  // (whole slices only: `kend` is not looked at)
+  __device__ __forceinline__ i32x4 load_piece(int k0, int, int j) const {
     const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)(base + (int64_t)k0 * 2), 0, -1, 0x00020000);
     return __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)off[j], 0, 0));
   }
@@ -293,8 +294,12 @@ struct TransOp {
     else load_to_lds16<STREAM>(base + (int64_t)k0 * ld, off[j], tile + wave_uniform_id() * 1024 + rnd(j) * NT * 16);
   }
   // the same piece into registers (not for gathered rows), and where it belongs in the LDS tile
-  __device__ __forceinline__ i32x4 load_piece(int k0, int j) const {
-    const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)(base + (int64_t)k0 * ld), 0, -1, 0x00020000);
+  // Contraction rows from `kend` on read as zeros: the buffer descriptor of the slice ends with row kend - 1
+  // (a row's pieces lie inside its first `ld` bytes).
+  __device__ __forceinline__ i32x4 load_piece(int k0, int kend, int j) const {
+    const int64_t span = (int64_t)(kend - k0) * ld;
+    const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(base + (int64_t)k0 * ld), 0, span < 0xffffffffLL ? (int)(unsigned)span : -1, 0x00020000);
     return __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)off[j], 0, 0));
   }
   __device__ __forceinline__ int piece_lds(int j) const { return (rnd(j) * NT + (int)threadIdx.x) * 16; }
@@ -467,84 +472,99 @@ __device__ __forceinline__ void mainloop(AOp& A, BOp& B, int klen, char* lds, bo
 //   one barrier per slice, after step 2: behind it the fragments of step 0 of slice kt + 1 are read while the
 //   MFMAs of step 3 run.
 // Whole 64-deep slices only, at least two of them (the launcher checks); loads past the end re-read the last slice.
-template <typename T, class TL, class AOp, class BOp, int P>
-__device__ __forceinline__ void rs_slice(const AOp& A, const BOp& B, char* lds, int kt, int last_k0, int wm, int wn,
-                                         f32x16 (&acc)[TL::FM][TL::FN], i32x4 (&g)[2][16],
-                                         i32x4 (&fa)[2][TL::FM], i32x4 (&fb)[2][TL::FN]) {
-  constexpr int STAGE = AOp::LDS_BYTES + BOp::LDS_BYTES;
+template <typename T, class TL, class AOp, class BOp, int P, int KS>
+__device__ __forceinline__ void rs_step(const AOp& A, const BOp& B, const char* __restrict__ cur, char* __restrict__ nxt,
+                                        int k2, int k3, int kend, int wm, int wn,
+                                        f32x16 (&acc)[TL::FM][TL::FN], i32x4 (&g)[2][16],
+                                        i32x4 (&fa)[2][TL::FM], i32x4 (&fb)[2][TL::FN]) {
   constexpr int FM = TL::FM, FN = TL::FN, NM = FM * FN;
-  constexpr int DR = FM * AOp::DS_PER_FRAG + FN * BOp::DS_PER_FRAG;      // fragment reads per step
-  static_assert(NM == 16 && DR >= 8 && DR <= 16, "pipeline below is laid out for 16 MFMAs per step");
-  char* cur = lds + P * STAGE;
-  char* nxt = lds + (P ^ 1) * STAGE;
+  static_assert(NM == 16 && FM + FN <= 8, "pipeline below is laid out for 16 MFMAs per step");
   constexpr int S = P ^ 1;
-  const int k2 = min((kt + 2) * BK, last_k0), k3 = min((kt + 3) * BK, last_k0);
+  constexpr int c = KS & 1, n = c ^ 1;
+  // LDS traffic of the step in the order it is to be issued in (the compiler keeps reads and writes of LDS in
+  // program order): one fragment of the next step behind each of the first FM + FN MFMAs - from the stage being
+  // multiplied, in step 3 from the stage just filled - and one piece written behind every third MFMA of steps 0-2
+  // (pieces 0-4, 5-10, 11-15).
+  constexpr int W0[5] = {0, 5, 11, 16, 16};
+  const char* src = KS < 3 ? cur : (const char*)nxt;
+  constexpr int fstep = KS < 3 ? KS + 1 : 0;
 #pragma unroll
-  for (int ks = 0; ks < 4; ++ks) {
-    const int c = ks & 1, n = c ^ 1;
-    const char* src = ks < 3 ? cur : nxt;
-    const int step = ks < 3 ? ks + 1 : 0;
-#pragma unroll
-    for (int i = 0; i < FM; ++i) fa[n][i] = AOp::frag(src, wm * TL::WTM + i * 32, step);
-#pragma unroll
-    for (int j = 0; j < FN; ++j) fb[n][j] = BOp::frag(src + AOp::LDS_BYTES, wn * TL::WTN + j * 32, step);
-#pragma unroll
-    for (int i = 0; i < FM; ++i)
-#pragma unroll
-      for (int j = 0; j < FN; ++j) acc[i][j] = Mfma<T>::run(fb[c][j], fa[c][i], acc[i][j]);
-    // pieces written in this step: 0-5, 6-10, 11-15, none
-    constexpr int W0[5] = {0, 6, 11, 16, 16};
-#pragma unroll
-    for (int q = W0[ks]; q < W0[ks + 1]; ++q) {
+  for (int m = 0; m < NM; ++m) {
+    if (m < FM) fa[n][m] = AOp::frag(src, wm * TL::WTM + m * 32, fstep);
+    else if (m < FM + FN) fb[n][m - FM] = BOp::frag(src + AOp::LDS_BYTES, wn * TL::WTN + (m - FM) * 32, fstep);
+    if ((KS * NM + m) % 3 == 1 && KS < 3) {
+      const int q = (KS * NM + m) / 3;
       if (q & 1) lds_write16(nxt + AOp::LDS_BYTES + B.piece_lds(q >> 1), g[S][q]);
       else lds_write16(nxt + A.piece_lds(q >> 1), g[S][q]);
     }
-    // pieces loaded in this step: 12-15 of the other set (slice kt + 2), then 0-3, 4-7, 8-11 of this one (slice kt + 3)
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int q = ks == 0 ? 12 + u : (ks - 1) * 4 + u;
-      const int k0 = ks == 0 ? k2 : k3;
-      i32x4& dst = ks == 0 ? g[P][q] : g[S][q];
-      dst = (q & 1) ? B.load_piece(k0, q >> 1) : A.load_piece(k0, q >> 1);
-    }
-#pragma unroll
-    for (int m = 0; m < NM; ++m) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      if (m < DR - 8) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-      else if (m < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      else if (m - 8 < W0[ks + 1] - W0[ks]) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-      if (m % 4 == 3) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    if (ks == 2) {
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // this thread's pieces are in LDS, its reads of `cur` done
-      __builtin_amdgcn_s_barrier();
-      __builtin_amdgcn_sched_barrier(0);
-    }
   }
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+#pragma unroll
+    for (int j = 0; j < FN; ++j) acc[i][j] = Mfma<T>::run(fb[c][j], fa[c][i], acc[i][j]);
+  static_assert(W0[1] == 5 && W0[2] == 11, "pieces per step follow from one write per three MFMAs");
+  // pieces loaded in this step: 12-15 of the other set (slice kt + 2), then 0-3, 4-7, 8-11 of this one (slice kt + 3)
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    constexpr int SET = KS == 0 ? P : S;
+    const int q = KS == 0 ? 12 + u : (KS - 1) * 4 + u;
+    const int k0 = KS == 0 ? k2 : k3;
+    g[SET][q] = (q & 1) ? B.load_piece(k0, kend, q >> 1) : A.load_piece(k0, kend, q >> 1);
+  }
+#pragma unroll
+  for (int m = 0; m < NM; ++m) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    if (m < FM) __builtin_amdgcn_sched_group_barrier(0x100, AOp::DS_PER_FRAG, 0);
+    else if (m < FM + FN) __builtin_amdgcn_sched_group_barrier(0x100, BOp::DS_PER_FRAG, 0);
+    if ((KS * NM + m) % 3 == 1 && KS < 3) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+    if (m % 4 == 3) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  if constexpr (KS == 2) {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // this thread's pieces are in LDS, its reads of `cur` done
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+template <typename T, class TL, class AOp, class BOp, int P>
+__device__ __forceinline__ void rs_slice(const AOp& A, const BOp& B, const char* cur, char* nxt,
+                                         int kt, int last_k0, int kend, int wm, int wn,
+                                         f32x16 (&acc)[TL::FM][TL::FN], i32x4 (&g)[2][16],
+                                         i32x4 (&fa)[2][TL::FM], i32x4 (&fb)[2][TL::FN]) {
+  const int k2 = min((kt + 2) * BK, last_k0), k3 = min((kt + 3) * BK, last_k0);
+  __builtin_amdgcn_sched_barrier(0);
+  rs_step<T, TL, AOp, BOp, P, 0>(A, B, cur, nxt, k2, k3, kend, wm, wn, acc, g, fa, fb);
+  rs_step<T, TL, AOp, BOp, P, 1>(A, B, cur, nxt, k2, k3, kend, wm, wn, acc, g, fa, fb);
+  rs_step<T, TL, AOp, BOp, P, 2>(A, B, cur, nxt, k2, k3, kend, wm, wn, acc, g, fa, fb);
+  rs_step<T, TL, AOp, BOp, P, 3>(A, B, cur, nxt, k2, k3, kend, wm, wn, acc, g, fa, fb);
 }
 
 template <typename T, class TL, class AOp, class BOp>
 __device__ __forceinline__ void mainloop_rs(const AOp& A, const BOp& B, int klen, char* lds,
                                             f32x16 (&acc)[TL::FM][TL::FN]) {
   static_assert(AOp::R == 8 && BOp::R == 8 && BK == 64, "16 pieces per thread and slice");
+  constexpr int STAGE = AOp::LDS_BYTES + BOp::LDS_BYTES;
   const int wave = threadIdx.x >> 6;
   const int wm = wave / TL::WN, wn = wave % TL::WN;
-  const int nk = klen / BK;
+  // A partial last slice only with operands that zero-fill (TransOp); without any contraction rows one slice of
+  // zeros is multiplied (no branch around the loop: 256 accumulator registers would have to be merged behind it).
+  const int nk = max(1, (klen + BK - 1) / BK);
   const int last_k0 = (nk - 1) * BK;
   i32x4 g[2][16];
   i32x4 fa[2][TL::FM], fb[2][TL::FN];
+  const int k1 = min(BK, last_k0), k2 = min(2 * BK, last_k0);
 #pragma unroll
-  for (int q = 0; q < 16; ++q) g[0][q] = (q & 1) ? B.load_piece(0, q >> 1) : A.load_piece(0, q >> 1);
+  for (int q = 0; q < 16; ++q) g[0][q] = (q & 1) ? B.load_piece(0, klen, q >> 1) : A.load_piece(0, klen, q >> 1);
 #pragma unroll
-  for (int q = 0; q < 16; ++q) g[1][q] = (q & 1) ? B.load_piece(min(BK, last_k0), q >> 1) : A.load_piece(min(BK, last_k0), q >> 1);
+  for (int q = 0; q < 16; ++q) g[1][q] = (q & 1) ? B.load_piece(k1, klen, q >> 1) : A.load_piece(k1, klen, q >> 1);
 #pragma unroll
   for (int q = 0; q < 16; ++q) {
     if (q & 1) lds_write16(lds + AOp::LDS_BYTES + B.piece_lds(q >> 1), g[0][q]);
     else lds_write16(lds + A.piece_lds(q >> 1), g[0][q]);
   }
 #pragma unroll
-  for (int q = 0; q < 12; ++q) g[0][q] = (q & 1) ? B.load_piece(min(2 * BK, last_k0), q >> 1) : A.load_piece(min(2 * BK, last_k0), q >> 1);
+  for (int q = 0; q < 12; ++q) g[0][q] = (q & 1) ? B.load_piece(k2, klen, q >> 1) : A.load_piece(k2, klen, q >> 1);
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_sched_barrier(0);
@@ -552,12 +572,18 @@ __device__ __forceinline__ void mainloop_rs(const AOp& A, const BOp& B, int klen
   for (int i = 0; i < TL::FM; ++i) fa[0][i] = AOp::frag(lds, wm * TL::WTM + i * 32, 0);
 #pragma unroll
   for (int j = 0; j < TL::FN; ++j) fb[0][j] = BOp::frag(lds + AOp::LDS_BYTES, wn * TL::WTN + j * 32, 0);
+  // The second stage starts 64 KB into LDS, beyond what the offset field of an LDS instruction can add: its
+  // addresses are formed from a base of their own (kept from being folded into constants), not with one
+  // vector-ALU instruction per access.
+  unsigned second = STAGE;
+  asm volatile("" : "+v"(second));
+  char* lds1 = lds + second;
   int kt = 0;
   for (; kt + 1 < nk; kt += 2) {
-    rs_slice<T, TL, AOp, BOp, 0>(A, B, lds, kt, last_k0, wm, wn, acc, g, fa, fb);
-    rs_slice<T, TL, AOp, BOp, 1>(A, B, lds, kt + 1, last_k0, wm, wn, acc, g, fa, fb);
+    rs_slice<T, TL, AOp, BOp, 0>(A, B, lds, lds1, kt, last_k0, klen, wm, wn, acc, g, fa, fb);
+    rs_slice<T, TL, AOp, BOp, 1>(A, B, lds1, lds, kt + 1, last_k0, klen, wm, wn, acc, g, fa, fb);
   }
-  if (kt < nk) rs_slice<T, TL, AOp, BOp, 0>(A, B, lds, kt, last_k0, wm, wn, acc, g, fa, fb);
+  if (kt < nk) rs_slice<T, TL, AOp, BOp, 0>(A, B, lds, lds1, kt, last_k0, klen, wm, wn, acc, g, fa, fb);
 }
 
 // Main loop of the small-row (decode) tile class: memory bound, so what matters is bytes in flight.  The
@@ -1304,12 +1330,13 @@ static int tail_split(const S2SArgs& a) {
 }
 
 // The 256 x 256 class.  Products with a long enough contraction run on the one-wave-per-SIMD form of it
-// (mainloop_rs: Mixtral shape, per 64-deep slice 2 420-2 550 cycles against 2 890-3 000; its prologue and its
+// (mainloop_rs: Mixtral shape, per 64-deep slice 2 300-2 420 cycles against 2 890-3 000; its prologue and its
 // epilogue, run by half as many threads, cost about 5 000 cycles more per tile, which a 12-slice contraction does not
 // earn back: K = 768 is 5 % slower, K = 1536 even, K = 2048 is 5-8 % faster).  The fused gated-unit gradient stays with
 // the 8-wave form: its epilogue is bound by vector-ALU work that 8 waves overlap better (Mixtral: 3.91 against 4.04 ms).
 // Both forms add up every output element in the same order: the same bits.
 static constexpr int RS_MIN_K = 1792;
+static constexpr int RS_XTY_MIN_ROWS = 3072;      // groupXtY: average rows per expert from which that form is used
 template <typename T>
 static int launch_main(const S2SArgs& a, bool b_tr, hipStream_t st) {
   bool al16 = true;             // the one-wave-per-SIMD form has only the LDS-staged epilogues (16-byte pieces)
@@ -1415,6 +1442,7 @@ __global__ __launch_bounds__(TL::NT) void xty_mfma_kernel(XtYPlan a, Raster rast
   __shared__ __attribute__((aligned(16))) char lds[2 * STAGE];
   __shared__ int64_t sDst[TL::BM];
   __shared__ unsigned sRows[2 * 64];       // row offsets of a gathered operand (see TransOp)
+  __shared__ __attribute__((aligned(16))) float sBias[TL::RS ? TL::BN : 4];
 
   int m_tile, n_tile, m_loc, n_loc;
   if (!rast.map(blockIdx.x, m_tile, n_tile, m_loc, n_loc)) return;
@@ -1446,10 +1474,11 @@ __global__ __launch_bounds__(TL::NT) void xty_mfma_kernel(XtYPlan a, Raster rast
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
   }
   const bool want_db = a.Db != nullptr && a.db_from_p && n_tile == 0;
-  mainloop<T, TL, AOp, BOp, true>(A, B, r_hi - r_lo, lds, want_db, acc, rs);
+  if constexpr (TL::RS) mainloop_rs<T, TL, AOp, BOp>(A, B, r_hi - r_lo, lds, acc);      // no bias gradient, no gather
+  else mainloop<T, TL, AOp, BOp, true>(A, B, r_hi - r_lo, lds, want_db, acc, rs);
 
-  if ((((uintptr_t)a.OUT & 15) == 0) && ((a.soe | a.sop | a.nq) & 7) == 0)
-    epilogue_staged<T, TL>(acc, (T*)a.OUT, sDst, q0, a.nq, nullptr, 0, lds);
+  if (TL::RS || ((((uintptr_t)a.OUT & 15) == 0) && ((a.soe | a.sop | a.nq) & 7) == 0))
+    epilogue_staged<T, TL>(acc, (T*)a.OUT, sDst, q0, a.nq, nullptr, 0, lds, sBias);
   else
     epilogue<T, TL>(acc, (T*)a.OUT, sDst, q0, a.nq, nullptr, 0);
 
@@ -1499,9 +1528,8 @@ __global__ __launch_bounds__(256) void colsum_kernel(const T* __restrict__ DY, i
   }
 }
 
-template <typename T>
+template <typename T, class TL>
 static int launch_xty(const XtYArgs& a, hipStream_t st) {
-  typedef Tile<256, 256, 2, 4> TL;
   XtYPlan p;
   const bool k_contig = a.sdwk == 1;     // output rows = N index
   if (k_contig) {
@@ -1523,7 +1551,8 @@ static int launch_xty(const XtYArgs& a, hipStream_t st) {
   const Raster r = make_raster((int64_t)a.E * p_tiles, q_tiles, GM_XTY);
   const int64_t grid = r.grid();
   if (grid > 0x7fffffffLL) { set_error("smoe_groupXtY: grid too large"); return SMOE_ERR_RANGE; }
-  if (a.idx == nullptr) hipLaunchKernelGGL((xty_mfma_kernel<T, TL, false, false>), dim3((unsigned)grid), dim3(TL::NT), 0, st, p, r, p_tiles);
+  if constexpr (TL::RS) hipLaunchKernelGGL((xty_mfma_kernel<T, TL, false, false>), dim3((unsigned)grid), dim3(TL::NT), 0, st, p, r, p_tiles);
+  else if (a.idx == nullptr) hipLaunchKernelGGL((xty_mfma_kernel<T, TL, false, false>), dim3((unsigned)grid), dim3(TL::NT), 0, st, p, r, p_tiles);
   else if (k_contig) hipLaunchKernelGGL((xty_mfma_kernel<T, TL, false, true>), dim3((unsigned)grid), dim3(TL::NT), 0, st, p, r, p_tiles);
   else hipLaunchKernelGGL((xty_mfma_kernel<T, TL, true, false>), dim3((unsigned)grid), dim3(TL::NT), 0, st, p, r, p_tiles);
   int rc = launch_status("xty_mfma_kernel");
@@ -1550,7 +1579,19 @@ bool try_xty_mfma(const XtYArgs& a, int dtype, hipStream_t st, int& rc) {
   // step: N = 1536 (Qwen-like, top-8) 9.12 -> 8.90 ms, N = 5760 (gpt-oss-like) 6.07 -> 6.03 ms, N = 28672 (Mixtral)
   // 31.3 -> 31.5 ms: wide layers keep the separate pass.
   if (a.idx != nullptr && a.N > XTY_GATHER_MAX_N) return false;
-  rc = dtype == SMOE_BF16 ? launch_xty<bf16_t>(a, st) : launch_xty<f16_t>(a, st);
+  // One-wave-per-SIMD form: needs the LDS-staged epilogue; no gathered operand, no bias gradient in the main loop.
+  // Both operands are read transposed (two LDS reads per fragment), which leaves less to win than in
+  // scatter2scatter: Mixtral shape (4096 rows per expert) 3.28 -> 3.12 and 6.35 -> 6.20 ms, 1024 rows per expert
+  // 1-5 % slower.
+  const bool out16 = (((uintptr_t)a.DW & 15) == 0) && ((a.sdwe | (a.sdwk == 1 ? a.sdwn : a.sdwk) | (a.sdwk == 1 ? a.K : a.N)) & 7) == 0;
+  const bool db_in_loop = a.Db != nullptr && a.sdwk == 1;
+  if (a.idx == nullptr && !db_in_loop && out16 && a.L / a.E >= RS_XTY_MIN_ROWS) {
+    typedef Tile<256, 256, 2, 2, 2, true> RSTile;
+    rc = dtype == SMOE_BF16 ? launch_xty<bf16_t, RSTile>(a, st) : launch_xty<f16_t, RSTile>(a, st);
+    return true;
+  }
+  typedef Tile<256, 256, 2, 4> XTile;
+  rc = dtype == SMOE_BF16 ? launch_xty<bf16_t, XTile>(a, st) : launch_xty<f16_t, XTile>(a, st);
   return true;
 }
 

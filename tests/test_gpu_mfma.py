@@ -122,6 +122,47 @@ def test_s2s_launch_split_by_tile_rows(T, skew, x_grouped, y_grouped, w_layout):
     assert torch.equal(got, torch.cat(halves, 1))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("w_layout", ["k_contig", "n_contig"])
+@pytest.mark.parametrize("x_grouped,y_grouped", [(False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("K", [1792, 1856])
+def test_s2s_long_contraction(K, x_grouped, y_grouped, w_layout, dtype):
+    """Contractions of 1792 and more run on the one-wave-per-SIMD form of the 256 x 256 class (operands through
+    registers, 28 and 29 slices: the loop handles two slices per trip): ragged tile rows, an expert without rows,
+    a partial tile column, bias."""
+    T, E, k, N = 1500, 4, 2, 520
+    experts, (eid, idx, off) = _routing(T, E, k, seed=K, skew=0.5, empty=(2,))
+    g = torch.Generator().manual_seed(K + 1)
+    fan = 1 if x_grouped else k
+    X = torch.randn(T * k // fan, K, generator=g).to(dtype)
+    Wp = (torch.randn(E, N, K, generator=g) * 0.05).to(dtype)
+    b = torch.randn(E, N, generator=g).to(dtype)
+    Wd = Wp.to(DEV).permute(0, 2, 1)
+    if w_layout == "n_contig":
+        Wd = Wd.contiguous()
+    want = oracle.scatter2scatter_ref(X.float(), Wp.permute(0, 2, 1).float(), eid, idx, fan, b.float(), x_grouped, y_grouped)
+    out = torch.full((T * k, N), float("nan"), dtype=dtype, device=DEV)
+    got = ops.scatter2scatter(X.to(DEV), Wd, eid.to(DEV), idx.to(DEV), fan, b=b.to(DEV), x_grouped=x_grouped,
+                              y_grouped=y_grouped, out=out, expert_offsets=off.to(DEV))
+    _close(got, want, scale=0.05 * K ** 0.5)
+
+
+def test_s2s_long_contraction_same_bits_as_column_halves():
+    """The one-wave-per-SIMD form and the 8-wave form add up every output element in the same order: a product
+    whose remainder of tile rows goes to a second launch of 256 x 128 tiles (8 waves) equals, bit for bit, the two
+    launches over its column halves, which are not split."""
+    T, E, k, K, N = 4200, 8, 2, 1792, 4096
+    experts, (eid, idx, off) = _routing(T, E, k, seed=3)
+    g = torch.Generator().manual_seed(4)
+    X = torch.randn(T, K, generator=g).bfloat16().to(DEV)
+    Wd = (torch.randn(E, N, K, generator=g) * 0.05).bfloat16().to(DEV).permute(0, 2, 1)
+    args = (eid.to(DEV), idx.to(DEV), k)
+    kw = dict(y_grouped=True, expert_offsets=off.to(DEV))
+    got = ops.scatter2scatter(X, Wd, *args, **kw)
+    halves = [ops.scatter2scatter(X, Wd[:, :, c:c + N // 2], *args, **kw) for c in (0, N // 2)]
+    assert torch.equal(got, torch.cat(halves, 1))
+
+
 def test_split_product_replays_from_a_graph():
     """A product that runs as two launches (see the test above), routing included, captured into a HIP graph and
     replayed on fresh inputs, with eager work between the replays: every replay equals the eager result."""
@@ -192,6 +233,32 @@ def test_xty(T, E, k, K, N, out_layout, dtype):
     _close(Db, Db_ref, scale=0.1 * rows ** 0.5)
     for e in (torch.diff(off, prepend=torch.zeros(1, dtype=torch.long)) == 0).nonzero().flatten().tolist():
         assert not DW[e].any() and not Db[e].any()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("out_layout,has_bias", [("param", False), ("plain", False), ("plain", True)])
+def test_xty_long_segments(out_layout, has_bias, dtype):
+    """From 3072 rows per expert on average the weight gradient runs on the one-wave-per-SIMD form (unless the bias
+    gradient rides along in the main loop): ragged segment lengths (the last slice of a segment is zero-filled by the
+    loads themselves), an expert without rows, partial tiles in both output directions."""
+    T, E, K, N = 13000, 4, 264, 520
+    experts, (eid, idx, off) = _routing(T, E, 1, seed=17, skew=0.7, empty=(1,))
+    g = torch.Generator().manual_seed(18)
+    X = torch.randn(T, K, generator=g).to(dtype)
+    DY = (torch.randn(T, N, generator=g) * 0.1).to(dtype)
+    DW_ref, Db_ref = oracle.group_bwd_W_ref(DY.float(), X.float(), off, E, has_bias=has_bias)
+    counts = torch.diff(off, prepend=torch.zeros(1, dtype=torch.long))
+    assert int(counts.min()) == 0 and int((counts % 64 != 0).sum()) >= 2
+    if out_layout == "param":
+        DW, Db = ops.group_bwd_W(DY.to(DEV), X.to(DEV), off.to(DEV), E, has_bias=has_bias)
+    else:
+        DW = torch.full((E, K, N), float("nan"), dtype=dtype, device=DEV)
+        Db = torch.full((E, N), float("nan"), dtype=dtype, device=DEV) if has_bias else None
+        ops._xty_launch(E, DW, Db, DY.to(DEV), X.to(DEV), off.to(DEV))
+    _close(DW, DW_ref, scale=0.1 * int(counts.max()) ** 0.5)
+    if has_bias:
+        _close(Db, Db_ref, scale=0.1 * int(counts.max()) ** 0.5)
+    assert not DW[1].any()
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
