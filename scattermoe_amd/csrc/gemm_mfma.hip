@@ -941,48 +941,65 @@ template <typename T, class TL>
 __device__ __forceinline__ void epilogue_glu_bwd_staged(const f32x16 (&acc)[TL::FM][TL::FN], const S2SArgs& a,
                                                         int row0, int rows, int n0, char* lds, float* sbias = nullptr) {
   typedef T T8 __attribute__((ext_vector_type(8)));
-  constexpr int CPR = TL::BN / 8, PIECES = TL::BM * CPR, PP = PIECES / TL::NT, GRP = PP < 4 ? PP : 4;
-  static_assert(PIECES % TL::NT == 0 && PP % GRP == 0, "pieces must divide evenly");
+  constexpr int CPR = TL::BN / 8, PIECES = TL::BM * CPR, PP = PIECES / TL::NT;
+  constexpr int GRP = PP >= 8 ? 4 : (PP >= 2 ? PP / 2 : 1);       // pieces per group, two groups in flight
+  static_assert(PIECES % TL::NT == 0 && (PP == 1 || PP % (2 * GRP) == 0), "pieces must divide evenly");
   stage_accumulators<T, TL>(acc, lds, [](int) { return 0.0f; }, sbias);
   const int F = a.N;
   const bool gf = (a.act & 1) != 0;
   const T* pre = (const T*)a.aux;
   T* dpre = (T*)a.Y;
-#pragma unroll 1
-  for (int q0 = 0; q0 < PP; q0 += GRP) {
-    T8 p1[GRP], p2[GRP], dh[GRP];
-    bool ok[GRP];
+  // The saved pre-activation of the next group of pieces is on its way while the current group is worked on (loads of
+  // rows and columns outside the tile's valid part are redirected to its first row / column and their results dropped).
+  T8 p1[2][GRP], p2[2][GRP];
+  auto fetch = [&](auto buf, int q0) {
 #pragma unroll
     for (int u = 0; u < GRP; ++u) {
       const int p = (q0 + u) * TL::NT + threadIdx.x;
-      const int row = p / CPR, c = p % CPR, n = n0 + c * 8;
-      ok[u] = row < rows && n < F;
-      if (ok[u]) {
-        const T* src = pre + (int64_t)(row0 + row) * a.saux + n;
-        p1[u] = *(const T8*)src;
-        p2[u] = *(const T8*)(src + F);
-      }
-      dh[u] = *(const T8*)(lds + staged_addr<TL>(row, c * 8));
+      const int row = p / CPR, n = n0 + (p % CPR) * 8;
+      const T* src = pre + (int64_t)(row0 + (row < rows ? row : 0)) * a.saux + (n < F ? n : 0);
+      p1[decltype(buf)::value][u] = *(const T8*)src;
+      p2[decltype(buf)::value][u] = *(const T8*)(src + F);
+    }
+  };
+  auto work = [&](auto buf, int q0) {
+    T8 dh[GRP];
+#pragma unroll
+    for (int u = 0; u < GRP; ++u) {
+      const int p = (q0 + u) * TL::NT + threadIdx.x;
+      dh[u] = *(const T8*)(lds + staged_addr<TL>(p / CPR, (p % CPR) * 8));
     }
 #pragma unroll
     for (int u = 0; u < GRP; ++u) {
-      if (!ok[u]) continue;
       const int p = (q0 + u) * TL::NT + threadIdx.x;
       const int row = p / CPR, n = n0 + (p % CPR) * 8;
       T8 o1, o2;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
+        const T v1 = p1[decltype(buf)::value][u][e], v2 = p2[decltype(buf)::value][u][e];
         const float dv = to_f32(dh[u][e]);
-        const float lin = to_f32(gf ? p2[u][e] : p1[u][e]), gat = to_f32(gf ? p1[u][e] : p2[u][e]);
+        const float lin = to_f32(gf ? v2 : v1), gat = to_f32(gf ? v1 : v2);
         float f_lin, f_gat;
-          glu_grad(a.act, dv, gat, lin, f_lin, f_gat);
-          const T d_lin = from_f32<T>(f_lin), d_gat = from_f32<T>(f_gat);
+        glu_grad(a.act, dv, gat, lin, f_lin, f_gat);
+        const T d_lin = from_f32<T>(f_lin), d_gat = from_f32<T>(f_gat);
         o1[e] = gf ? d_gat : d_lin;
         o2[e] = gf ? d_lin : d_gat;
       }
-      T* dst = dpre + (int64_t)(row0 + row) * a.sym + n;
-      stream_store(o1, (T8*)dst);
-      stream_store(o2, (T8*)(dst + F));
+      if (row < rows && n < F) {
+        T* dst = dpre + (int64_t)(row0 + row) * a.sym + n;
+        stream_store(o1, (T8*)dst);
+        stream_store(o2, (T8*)(dst + F));
+      }
+    }
+  };
+  fetch(std::integral_constant<int, 0>(), 0);
+#pragma unroll 1
+  for (int q0 = 0; q0 < PP; q0 += 2 * GRP) {
+    if constexpr (PP > 1) fetch(std::integral_constant<int, 1>(), q0 + GRP);
+    work(std::integral_constant<int, 0>(), q0);
+    if constexpr (PP > 1) {
+      if (q0 + 2 * GRP < PP) fetch(std::integral_constant<int, 0>(), q0 + 2 * GRP);
+      work(std::integral_constant<int, 1>(), q0 + GRP);
     }
   }
 }
@@ -1024,47 +1041,63 @@ template <typename T, class TL>
 __device__ __forceinline__ void epilogue_oss_bwd_staged(const f32x16 (&acc)[TL::FM][TL::FN], const S2SArgs& a,
                                                         int row0, int rows, int n0, char* lds, float* sbias = nullptr) {
   typedef T T8 __attribute__((ext_vector_type(8)));
-  constexpr int CPR = TL::BN / 8, PIECES = TL::BM * CPR, PP = PIECES / TL::NT, GRP = PP < 4 ? PP : 4;
-  static_assert(PIECES % TL::NT == 0 && PP % GRP == 0, "pieces must divide evenly");
+  constexpr int CPR = TL::BN / 8, PIECES = TL::BM * CPR, PP = PIECES / TL::NT;
+  constexpr int GRP = PP >= 8 ? 4 : (PP >= 2 ? PP / 2 : 1);       // pieces per group, two groups in flight
+  static_assert(PIECES % TL::NT == 0 && (PP == 1 || PP % (2 * GRP) == 0), "pieces must divide evenly");
   stage_accumulators<T, TL>(acc, lds, [](int) { return 0.0f; }, sbias);
   const int F = a.N;
   const T* pre = (const T*)a.aux;
   T* dpre = (T*)a.Y;
-#pragma unroll 1
-  for (int q0 = 0; q0 < PP; q0 += GRP) {
-    T8 p1[GRP], p2[GRP], dh[GRP];
-    bool ok[GRP];
+  // next group's saved pre-activation pairs on their way while the current group is worked on (see epilogue_glu_bwd_staged)
+  T8 p1[2][GRP], p2[2][GRP];
+  auto fetch = [&](auto buf, int q0) {
 #pragma unroll
     for (int u = 0; u < GRP; ++u) {
       const int p = (q0 + u) * TL::NT + threadIdx.x;
-      const int row = p / CPR, c = p % CPR, n = n0 + c * 8;
-      ok[u] = row < rows && n < F;
-      if (ok[u]) {
-        const T* src = pre + (int64_t)(row0 + row) * a.saux + 2 * n;
-        p1[u] = *(const T8*)src;
-        p2[u] = *(const T8*)(src + 8);
-      }
-      dh[u] = *(const T8*)(lds + staged_addr<TL>(row, c * 8));
+      const int row = p / CPR, n = n0 + (p % CPR) * 8;
+      const T* src = pre + (int64_t)(row0 + (row < rows ? row : 0)) * a.saux + 2 * (n < F ? n : 0);
+      p1[decltype(buf)::value][u] = *(const T8*)src;
+      p2[decltype(buf)::value][u] = *(const T8*)(src + 8);
+    }
+  };
+  auto work = [&](auto buf, int q0) {
+    T8 dh[GRP];
+#pragma unroll
+    for (int u = 0; u < GRP; ++u) {
+      const int p = (q0 + u) * TL::NT + threadIdx.x;
+      dh[u] = *(const T8*)(lds + staged_addr<TL>(p / CPR, (p % CPR) * 8));
     }
 #pragma unroll
     for (int u = 0; u < GRP; ++u) {
-      if (!ok[u]) continue;
       const int p = (q0 + u) * TL::NT + threadIdx.x;
       const int row = p / CPR, n = n0 + (p % CPR) * 8;
+      const T8 v1 = p1[decltype(buf)::value][u], v2 = p2[decltype(buf)::value][u];
       T8 o1, o2;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         float dg, du;
-        oss_grad(to_f32(p1[u][2 * e]), to_f32(p1[u][2 * e + 1]), to_f32(dh[u][e]), a.alpha, a.limit, dg, du);
+        oss_grad(to_f32(v1[2 * e]), to_f32(v1[2 * e + 1]), to_f32(dh[u][e]), a.alpha, a.limit, dg, du);
         o1[2 * e] = from_f32<T>(dg);
         o1[2 * e + 1] = from_f32<T>(du);
-        oss_grad(to_f32(p2[u][2 * e]), to_f32(p2[u][2 * e + 1]), to_f32(dh[u][4 + e]), a.alpha, a.limit, dg, du);
+        oss_grad(to_f32(v2[2 * e]), to_f32(v2[2 * e + 1]), to_f32(dh[u][4 + e]), a.alpha, a.limit, dg, du);
         o2[2 * e] = from_f32<T>(dg);
         o2[2 * e + 1] = from_f32<T>(du);
       }
-      T* dst = dpre + (int64_t)(row0 + row) * a.sym + 2 * n;
-      stream_store(o1, (T8*)dst);
-      stream_store(o2, (T8*)(dst + 8));
+      if (row < rows && n < F) {
+        T* dst = dpre + (int64_t)(row0 + row) * a.sym + 2 * n;
+        stream_store(o1, (T8*)dst);
+        stream_store(o2, (T8*)(dst + 8));
+      }
+    }
+  };
+  fetch(std::integral_constant<int, 0>(), 0);
+#pragma unroll 1
+  for (int q0 = 0; q0 < PP; q0 += 2 * GRP) {
+    if constexpr (PP > 1) fetch(std::integral_constant<int, 1>(), q0 + GRP);
+    work(std::integral_constant<int, 0>(), q0);
+    if constexpr (PP > 1) {
+      if (q0 + 2 * GRP < PP) fetch(std::integral_constant<int, 0>(), q0 + 2 * GRP);
+      work(std::integral_constant<int, 1>(), q0 + GRP);
     }
   }
 }
@@ -1332,8 +1365,7 @@ static int tail_split(const S2SArgs& a) {
 // The 256 x 256 class.  Products with a long enough contraction run on the one-wave-per-SIMD form of it
 // (mainloop_rs: Mixtral shape, per 64-deep slice 2 300-2 420 cycles against 2 890-3 000; its prologue and its
 // epilogue, run by half as many threads, cost about 5 000 cycles more per tile, which a 12-slice contraction does not
-// earn back: K = 768 is 5 % slower, K = 1536 even, K = 2048 is 5-8 % faster).  The fused gated-unit gradient stays with
-// the 8-wave form: its epilogue is bound by vector-ALU work that 8 waves overlap better (Mixtral: 3.91 against 4.04 ms).
+// earn back: K = 768 is 5 % slower, K = 1536 even, K = 2048 is 5-8 % faster).
 // Both forms add up every output element in the same order: the same bits.
 static constexpr int RS_MIN_K = 1792;
 static constexpr int RS_XTY_MIN_ROWS = 3072;      // groupXtY: average rows per expert from which that form is used
@@ -1342,7 +1374,8 @@ static int launch_main(const S2SArgs& a, bool b_tr, hipStream_t st) {
   bool al16 = true;             // the one-wave-per-SIMD form has only the LDS-staged epilogues (16-byte pieces)
   if (a.glu == 0) al16 = (((uintptr_t)a.Y & 15) == 0) && ((a.sym | a.N) & 7) == 0;
   else if (a.glu == 1) al16 = ((((uintptr_t)a.Y | (uintptr_t)a.H) & 15) == 0) && ((a.sym | a.shm | a.N) & 7) == 0;
-  if (al16 && a.glu != 2 && a.glu != 4 && a.K % BK == 0 && a.K >= RS_MIN_K)
+  else if (a.glu == 2) al16 = ((((uintptr_t)a.aux | (uintptr_t)a.Y) & 15) == 0) && ((a.saux | a.sym | a.N) & 7) == 0;
+  if (al16 && a.K % BK == 0 && a.K >= RS_MIN_K)
     return launch_s2s<T, Tile<256, 256, 2, 2, 2, true>>(a, b_tr, st);
   return launch_s2s<T, Tile<256, 256, 2, 4>>(a, b_tr, st);
 }
