@@ -103,9 +103,11 @@ __device__ __forceinline__ void oss_grad(float gate, float up, float dh, float a
 // Every wave of the block runs this redundantly and gets the same (uniform) answer.
 // Returns false when `t` is past the last tile (the grid is sized by the host-known upper bound
 // floor(L/BM) + E, so surplus blocks simply exit).
+// `skip_small` > 0: an expert's last, partly filled tile is left out when it holds at most `skip_small` rows (another
+// launch with lower tiles takes those rows, see find_remainder).
 template <int BM>
 __device__ __forceinline__ bool find_tile(const int64_t* __restrict__ off, int E, int t,
-                                          int& expert, int& row_start, int& rows) {
+                                          int& expert, int& row_start, int& rows, int skip_small = 0) {
   const int lane = lane_id();
   int tiles_before = 0;
   for (int e0 = 0; e0 < E; e0 += 64) {
@@ -115,7 +117,9 @@ __device__ __forceinline__ bool find_tile(const int64_t* __restrict__ off, int E
       hi = (int)off[e];
       lo = e ? (int)off[e - 1] : 0;
     }
-    const int nt = (hi - lo + BM - 1) / BM;
+    int nt = (hi - lo + BM - 1) / BM;
+    const int rem = (hi - lo) % BM;
+    if (rem != 0 && rem <= skip_small) nt -= 1;
     int incl = nt;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
@@ -136,6 +140,20 @@ __device__ __forceinline__ bool find_tile(const int64_t* __restrict__ off, int E
     tiles_before += __shfl(incl, 63, 64);
   }
   return false;
+}
+
+// The rows that find_tile<BM>(..., skip_small) leaves out, as one tile per expert: the last n % BM rows of expert e
+// when there are between 1 and `small` of them.
+template <int BM>
+__device__ __forceinline__ bool find_remainder(const int64_t* __restrict__ off, int E, int e, int small,
+                                               int& row_start, int& rows) {
+  if (e >= E) return false;
+  const int hi = (int)off[e], lo = e ? (int)off[e - 1] : 0;
+  const int rem = (hi - lo) % BM;
+  if (rem == 0 || rem > small) return false;
+  row_start = hi - rem;
+  rows = rem;
+  return true;
 }
 
 static inline int64_t cdiv64(int64_t a, int64_t b) { return (a + b - 1) / b; }
@@ -170,6 +188,9 @@ struct S2SArgs {
   // Part of a product split by tile rows (MFMA path only): the launch covers the tile rows
   // [m_begin, m_begin + m_count) of its tile height.
   int m_begin = 0, m_count = 0x7fffffff;
+  // Products whose experts end in a partly filled tile (MFMA path only).  1: this launch leaves out every expert's
+  // last tile when it holds at most 128 rows; 2: this launch takes exactly those rows, one tile row per expert.
+  int tail_mode = 0;
 };
 
 struct XtYArgs {

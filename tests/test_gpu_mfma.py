@@ -163,6 +163,79 @@ def test_s2s_long_contraction_same_bits_as_column_halves():
     assert torch.equal(got, torch.cat(halves, 1))
 
 
+LAST_TILE_COUNTS = [1380, 1224, 1024, 0, 60, 1408, 1409, 1281]
+
+
+def _routing_with_counts(counts, k, seed):
+    """Routing in which expert e receives exactly counts[e] of the T * k slots."""
+    E, L = len(counts), sum(counts)
+    g = torch.Generator().manual_seed(seed)
+    experts = torch.repeat_interleave(torch.arange(E), torch.tensor(counts))[torch.randperm(L, generator=g)].view(L // k, k)
+    eid, idx, off = oracle.route_ref(experts, E)
+    assert off.tolist() == torch.tensor(counts).cumsum(0).tolist()
+    return eid, idx, off, g
+
+
+@pytest.mark.parametrize("x_grouped,y_grouped", [(False, True), (True, False), (True, True)])
+def test_s2s_last_tiles_of_few_rows_in_their_own_launch(x_grouped, y_grouped):
+    """A large product with fewer than 1536 rows per expert leaves every expert's last tile of at most 128 rows to a
+    second launch of 128-row tiles.  Row counts chosen for each case of the tile lookup: a last tile of 100 rows
+    (second launch), of 200 rows (stays), none (exact multiple of 256), an expert without rows, one of 60 rows
+    (only the second launch sees it), last tiles of exactly 128 and of 129 rows, and one of 1 row.  Every row must
+    be written once, to the oracle's values, and with the same bits as the launches over the column halves, which
+    are too small to be split.  (30 tile columns: 3.75 rounds, so the product is not cut by whole rounds instead.)"""
+    counts, k, K, N = LAST_TILE_COUNTS, 2, 2048, 7680
+    E, L = len(counts), sum(counts)
+    eid, idx, off, g = _routing_with_counts(counts, k, seed=11)
+    fan = 1 if x_grouped else k
+    X = torch.randn(L // fan, K, generator=g).bfloat16()
+    Wp = (torch.randn(E, N, K, generator=g) * 0.05).bfloat16()
+    b = torch.randn(E, N, generator=g).bfloat16()
+    Wd = Wp.to(DEV).permute(0, 2, 1)
+    args = (eid.to(DEV), idx.to(DEV), fan)
+    kw = dict(x_grouped=x_grouped, y_grouped=y_grouped, expert_offsets=off.to(DEV))
+    out = torch.full((L, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    got = ops.scatter2scatter(X.to(DEV), Wd, *args, b=b.to(DEV), out=out, **kw)
+    want = oracle.scatter2scatter_ref(X.float(), Wp.permute(0, 2, 1).float(), eid, idx, fan, b.float(), x_grouped, y_grouped)
+    _close(got, want, scale=0.05 * K ** 0.5)
+    halves = [ops.scatter2scatter(X.to(DEV), Wd[:, :, c:c + N // 2], *args, b=b.to(DEV)[:, c:c + N // 2], **kw)
+              for c in (0, N // 2)]
+    assert torch.equal(got, torch.cat(halves, 1))
+
+
+@pytest.mark.parametrize("act", ["SILU", "GPT_OSS"])
+def test_fused_gated_products_with_last_tiles_in_their_own_launch(act):
+    """The same row counts through the products that carry the gated unit in their epilogue (forward: saved
+    pre-activations and hidden rows; backward: gradient of the pre-activations), against the plain product followed
+    by the elementwise pass, which is checked above."""
+    counts, k, d, F = LAST_TILE_COUNTS, 2, 2048, 4096
+    E, L = len(counts), sum(counts)
+    eid, idx, off, g = _routing_with_counts(counts, k, seed=12)
+    eid, idx, off = eid.to(DEV), idx.to(DEV), off.to(DEV)
+    code = getattr(ops, "ACT_" + act)
+    extra = dict(alpha=1.702, limit=7.0) if act == "GPT_OSS" else {}
+    x = torch.randn(L // k, d, generator=g).bfloat16().to(DEV)
+    W1 = (torch.randn(E, 2 * F, d, generator=g) * 0.05).bfloat16().to(DEV).permute(0, 2, 1)
+    b1 = (torch.randn(E, 2 * F, generator=g) * 0.1).bfloat16().to(DEV)
+    pre_ref = ops.scatter2scatter(x, W1, eid, idx, k, b=b1, y_grouped=True, expert_offsets=off)
+    pre, h = ops.scatter2scatter_glu(x, W1, eid, idx, k, b=b1, act=code, expert_offsets=off, **extra)
+    assert torch.equal(pre, pre_ref)
+    h_ref = ops.gpt_oss_glu(pre_ref, 1.702, 7.0) if act == "GPT_OSS" else ops.glu_fwd(pre_ref, code)
+    assert float((h.float() - h_ref.float()).abs().max()) <= 2 ** -7 * float(h_ref.float().abs().max())
+    # backward through the second linear: (L, d) gradient rows times (E, d, F) weights, 2 * L * d * F flop
+    dy = torch.randn(L, 2 * d, generator=g).bfloat16().to(DEV)
+    W2 = (torch.randn(E, 2 * d, F, generator=g) * 0.05).bfloat16().to(DEV)
+    dh = ops.scatter2scatter(dy, W2, eid, idx, 1, x_grouped=True, y_grouped=True, expert_offsets=off)
+    ref = torch.empty_like(pre)
+    if act == "GPT_OSS":
+        ops._launch("oss_glu_bwd", pre, dh, ref, 1.702, 7.0)
+    else:
+        ref = ops.glu_bwd(pre, dh, code)
+    got = ops.scatter2scatter_glu_bwd(dy, W2, pre, eid, idx, act=code, expert_offsets=off, **extra)
+    err = (got.float() - ref.float()).abs()
+    assert bool((err <= 2 ** -7 * ref.float().abs() + 1e-30).all())
+
+
 def test_split_product_replays_from_a_graph():
     """A product that runs as two launches (see the test above), routing included, captured into a HIP graph and
     replayed on fresh inputs, with eager work between the replays: every replay equals the eager result."""
