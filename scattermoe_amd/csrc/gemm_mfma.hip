@@ -884,12 +884,28 @@ __device__ __forceinline__ void epilogue_staged(const f32x16 (&acc)[TL::FM][TL::
   stage_accumulators<T, TL>(acc, lds, [&](int tc) {
     return bias != nullptr && n0 + tc < ncols ? to_f32(bias[(int64_t)(n0 + tc) * sb]) : 0.0f;
   }, sbias);
+  // In groups: the row offsets of a group, then its pieces, are read from LDS back to back before the first of its
+  // stores (written as one conditional store per piece, every piece would wait for two LDS round trips of its own)
+  constexpr int GRP = PP >= 16 ? 16 : PP;
+  static_assert(PP % GRP == 0, "groups must divide the pieces");
 #pragma unroll
-  for (int q = 0; q < PP; ++q) {
-    const int p = q * TL::NT + threadIdx.x;
-    const int row = p / CPR, c = p % CPR, n = n0 + c * 8;
-    const int64_t d = dst[row];
-    if (d >= 0 && n < ncols) stream_store(*(const T8*)(lds + staged_addr<TL>(row, c * 8)), (T8*)(out + d + n));
+  for (int q0 = 0; q0 < PP; q0 += GRP) {
+    int64_t d[GRP];
+    T8 v[GRP];
+#pragma unroll
+    for (int g = 0; g < GRP; ++g) d[g] = dst[((q0 + g) * TL::NT + threadIdx.x) / CPR];
+#pragma unroll
+    for (int g = 0; g < GRP; ++g) {
+      const int p = (q0 + g) * TL::NT + threadIdx.x;
+      v[g] = *(const T8*)(lds + staged_addr<TL>(p / CPR, (p % CPR) * 8));
+    }
+#pragma unroll
+    for (int g = 0; g < GRP; ++g) asm volatile("" : "+v"(v[g]), "+v"(d[g]));      // keeps the reads above the branches
+#pragma unroll
+    for (int g = 0; g < GRP; ++g) {
+      const int n = n0 + (((q0 + g) * TL::NT + threadIdx.x) % CPR) * 8;
+      if (d[g] >= 0 && n < ncols) stream_store(v[g], (T8*)(out + d[g] + n));
+    }
   }
 }
 
@@ -913,25 +929,39 @@ __device__ __forceinline__ void epilogue_glu_fwd_staged(const f32x16 (&acc)[TL::
     const bool gf = (a.act & 1) != 0;
     T* pre = (T*)a.Y;
     T* hid = (T*)a.H;
+    // a group's LDS reads are issued back to back ahead of its arithmetic and stores (see epilogue_staged)
+    constexpr int GRP = PP >= 8 ? 8 : PP;
+    static_assert(PP % GRP == 0, "groups must divide the pieces");
 #pragma unroll
-    for (int q = 0; q < PP; ++q) {
-      const int p = q * TL::NT + threadIdx.x;
-      const int row = p / CPR, hc = (p % CPR) * 8;            // hidden column inside the tile
-      const int n = nh0 + hc;
-      if (row >= rows || n >= F) continue;
-      const int tc = (hc / HALF) * TL::WTN + hc % HALF;       // tile column of the first-half value
-      const T8 first = *(const T8*)(lds + staged_addr<TL>(row, tc));
-      const T8 second = *(const T8*)(lds + staged_addr<TL>(row, tc + HALF));
-      T8 h;
+    for (int q0 = 0; q0 < PP; q0 += GRP) {
+      T8 v1[GRP], v2[GRP];
 #pragma unroll
-      for (int e = 0; e < 8; ++e)
-        h[e] = from_f32<T>(glu_h(a.act, to_f32(gf ? first[e] : second[e]), to_f32(gf ? second[e] : first[e])));
-      const int64_t r = row0 + row;
-      if (pre != nullptr) {
-        stream_store(first, (T8*)(pre + r * a.sym + n));
-        stream_store(second, (T8*)(pre + r * a.sym + F + n));
+      for (int g = 0; g < GRP; ++g) {
+        const int p = (q0 + g) * TL::NT + threadIdx.x;
+        const int row = p / CPR, hc = (p % CPR) * 8;          // hidden column inside the tile
+        const int tc = (hc / HALF) * TL::WTN + hc % HALF;     // tile column of the first-half value
+        v1[g] = *(const T8*)(lds + staged_addr<TL>(row, tc));
+        v2[g] = *(const T8*)(lds + staged_addr<TL>(row, tc + HALF));
       }
-      stream_store(h, (T8*)(hid + r * a.shm + n));
+#pragma unroll
+      for (int g = 0; g < GRP; ++g) asm volatile("" : "+v"(v1[g]), "+v"(v2[g]));
+#pragma unroll
+      for (int g = 0; g < GRP; ++g) {
+        const int p = (q0 + g) * TL::NT + threadIdx.x;
+        const int row = p / CPR, n = nh0 + (p % CPR) * 8;
+        if (row >= rows || n >= F) continue;
+        const T8 first = v1[g], second = v2[g];
+        T8 h;
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          h[e] = from_f32<T>(glu_h(a.act, to_f32(gf ? first[e] : second[e]), to_f32(gf ? second[e] : first[e])));
+        const int64_t r = row0 + row;
+        if (pre != nullptr) {
+          stream_store(first, (T8*)(pre + r * a.sym + n));
+          stream_store(second, (T8*)(pre + r * a.sym + F + n));
+        }
+        stream_store(h, (T8*)(hid + r * a.shm + n));
+      }
     }
   }
 }
@@ -1021,18 +1051,31 @@ __device__ __forceinline__ void epilogue_oss_fwd_staged(const f32x16 (&acc)[TL::
   }, sbias);
   T* pre = (T*)a.Y;
   T* hid = (T*)a.H;
+  constexpr int GRP = PP >= 16 ? 16 : PP;               // LDS reads of a group back to back (see epilogue_staged)
+  static_assert(PP % GRP == 0, "groups must divide the pieces");
 #pragma unroll
-  for (int q = 0; q < PP; ++q) {
-    const int p = q * TL::NT + threadIdx.x;
-    const int row = p / CPR, c = p % CPR, n = n0 + c * 8;
-    if (row >= rows || n >= a.N) continue;
-    const T8 v = *(const T8*)(lds + staged_addr<TL>(row, c * 8));
-    T4 h;
+  for (int q0 = 0; q0 < PP; q0 += GRP) {
+    T8 vs[GRP];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) h[e] = from_f32<T>(oss_h(to_f32(v[2 * e]), to_f32(v[2 * e + 1]), a.alpha, a.limit));
-    const int64_t r = row0 + row;
-    if (pre != nullptr) stream_store(v, (T8*)(pre + r * a.sym + n));
-    stream_store(h, (T4*)(hid + r * a.shm + n / 2));
+    for (int g = 0; g < GRP; ++g) {
+      const int p = (q0 + g) * TL::NT + threadIdx.x;
+      vs[g] = *(const T8*)(lds + staged_addr<TL>(p / CPR, (p % CPR) * 8));
+    }
+#pragma unroll
+    for (int g = 0; g < GRP; ++g) asm volatile("" : "+v"(vs[g]));
+#pragma unroll
+    for (int g = 0; g < GRP; ++g) {
+      const int p = (q0 + g) * TL::NT + threadIdx.x;
+      const int row = p / CPR, n = n0 + (p % CPR) * 8;
+      if (row >= rows || n >= a.N) continue;
+      const T8 v = vs[g];
+      T4 h;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) h[e] = from_f32<T>(oss_h(to_f32(v[2 * e]), to_f32(v[2 * e + 1]), a.alpha, a.limit));
+      const int64_t r = row0 + row;
+      if (pre != nullptr) stream_store(v, (T8*)(pre + r * a.sym + n));
+      stream_store(h, (T4*)(hid + r * a.shm + n / 2));
+    }
   }
 }
 
