@@ -1419,7 +1419,7 @@ static int tail_split(const S2SArgs& a) {
 // earn back: K = 768 is 5 % slower, K = 1536 even, K = 2048 is 5-8 % faster).
 // Both forms add up every output element in the same order: the same bits.
 static constexpr int RS_MIN_K = 1792;
-static constexpr int RS_XTY_MIN_ROWS = 3072;      // groupXtY: average rows per expert from which that form is used
+static constexpr int RS_XTY_MIN_ROWS = 2048;      // groupXtY: average rows per expert from which that form is used
 template <typename T>
 static int launch_main_class(const S2SArgs& a, bool b_tr, hipStream_t st) {
   bool al16 = true;             // the one-wave-per-SIMD form has only the LDS-staged epilogues (16-byte pieces)
@@ -1688,8 +1688,8 @@ bool try_xty_mfma(const XtYArgs& a, int dtype, hipStream_t st, int& rc) {
   if (a.idx != nullptr && a.N > XTY_GATHER_MAX_N) return false;
   // One-wave-per-SIMD form: needs the LDS-staged epilogue; no gathered operand, no bias gradient in the main loop.
   // Both operands are read transposed (two LDS reads per fragment), which leaves less to win than in
-  // scatter2scatter: Mixtral shape (4096 rows per expert) 3.28 -> 3.12 and 6.35 -> 6.20 ms, 1024 rows per expert
-  // 1-5 % slower.
+  // scatter2scatter: Mixtral shape (4096 rows per expert) 3.28 -> 3.12 and 6.35 -> 6.20 ms, 2048 rows per expert
+  // (128 experts, 768 x 2048 and 2048 x 1536 outputs) 0.81 -> 0.77 and 1.55 -> 1.51 ms, 1024 rows per expert even.
   const bool out16 = (((uintptr_t)a.DW & 15) == 0) && ((a.sdwe | (a.sdwk == 1 ? a.sdwn : a.sdwk) | (a.sdwk == 1 ? a.K : a.N)) & 7) == 0;
   const bool db_in_loop = a.Db != nullptr && a.sdwk == 1;
   if (a.idx == nullptr && !db_in_loop && out16 && a.L / a.E >= RS_XTY_MIN_ROWS) {

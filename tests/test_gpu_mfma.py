@@ -311,7 +311,7 @@ def test_xty(T, E, k, K, N, out_layout, dtype):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("out_layout,has_bias", [("param", False), ("plain", False), ("plain", True)])
 def test_xty_long_segments(out_layout, has_bias, dtype):
-    """From 3072 rows per expert on average the weight gradient runs on the one-wave-per-SIMD form (unless the bias
+    """From 2048 rows per expert on average the weight gradient runs on the one-wave-per-SIMD form (unless the bias
     gradient rides along in the main loop): ragged segment lengths (the last slice of a segment is zero-filled by the
     loads themselves), an expert without rows, partial tiles in both output directions."""
     T, E, K, N = 13000, 4, 264, 520
