@@ -270,6 +270,28 @@ def decode_line(args, cfg, torch):
                          hit, 3 if cfg.glu else 2)}}))
 
 
+def mfma_sustained(torch, lib):
+    """What the matrix pipe sustains on its own (no memory traffic), for all-zero operands and for operands with
+    random signs and mantissas: the shader clock follows the operand bits, so the nominal peak that `roofline.frac`
+    is priced against is not reachable on data that is not trivial."""
+    import ctypes
+    out = torch.empty(65536, dtype=torch.float32, device="cuda:0")
+    flop = ctypes.c_double(0.0)
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    res = {}
+    for name, kind in (("zero_operands", 0), ("random_operands", 1)):
+        for iters in (2000, 16000):                  # a short launch to settle the clock, then about 15 ms
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            rc = lib.smoe_mfma_rate_probe(ctypes.c_void_p(out.data_ptr()), iters, kind, ctypes.byref(flop), st)
+            b.record()
+            torch.cuda.synchronize()
+            assert rc == 0, "smoe_mfma_rate_probe failed: %d" % rc
+        res[name + "_tflops"] = round(flop.value / a.elapsed_time(b) / 1e9, 1)
+    res["kernel"] = "independent 32x32x16 bf16 MFMAs, one wave per SIMD on every CU, operands in registers"
+    return res
+
+
 def main():
     args = parse()
     if args.traffic_record:
@@ -353,6 +375,7 @@ def main():
     k_fl = sum(fl for _, fl in sel) / len(sel)
     achieved = k_fl / (k_ms * 1e-3) / 1e12
     traffic, traffic_src = measured_traffic(cfg.name, _C.source_hash())
+    sustained = mfma_sustained(torch, _C.load())
     roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": traffic, "traffic_source": traffic_src,
                 "kernel": "s2s_mfma_kernel (scatter2scatter products with K-contiguous weights; a product of a few "
@@ -371,6 +394,7 @@ def main():
             "tokens": cfg.T, "rows": L},
         "tflops": round(tflops, 1), "frac_of_bf16_mfma_peak": round(tflops / PEAK_BF16_TFLOPS, 4),
         "roofline": roofline,
+        "mfma_sustained": sustained,
         "products": products,
         "inputs": "router logits, X, dY: CPU generator seed 0 (tests/_inputs.make_inputs order); weights: device "
                   "generator seed 1, N(0, 0.02) (tests/_inputs.make_module)",

@@ -284,6 +284,16 @@ int smoe_topk_softmax(const void* logits, int64_t slt, int64_t sle, int64_t T, i
                       float* weights_out, int64_t swt, int64_t swk, int64_t* idx_out, int64_t sit, int64_t sik,
                       int dtype, void* stream);
 
+/*
+ * Measurement aid, no counterpart in the reference and no part of the MoE path: launches a kernel of nothing but
+ * independent 32x32x16 bf16 MFMAs (one wave per SIMD on every CU, operands in registers, no memory traffic) and
+ * stores the flop count of the launch in *flop_out.  `random_operands` = 0: all-zero operands; 1: random signs and
+ * mantissas.  The time of the launch (events on `stream`) gives the rate the matrix pipe sustains at the shader
+ * clock the power management grants for such operands; bench.py reports it beside the roofline fraction, which is
+ * priced against the nominal peak.  `out`: 65536 floats of device memory (overwritten).
+ */
+int smoe_mfma_rate_probe(float* out, int iters, int random_operands, double* flop_out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -13,7 +13,7 @@ CSRC = os.path.join(PKG_DIR, "csrc")
 OBJ_DIR = os.path.join(CSRC, "build")
 LIB_PATH = os.path.join(PKG_DIR, "libscattermoe_amd.so")
 
-SOURCES = ["capi.hip", "route.hip", "group.hip", "s2s_generic.hip", "xty_generic.hip", "gemm_mfma.hip", "fused.hip", "router.hip", "s2s_rowdot.hip", "gemm_f32.hip"]
+SOURCES = ["capi.hip", "route.hip", "group.hip", "s2s_generic.hip", "xty_generic.hip", "gemm_mfma.hip", "fused.hip", "router.hip", "s2s_rowdot.hip", "gemm_f32.hip", "mfma_probe.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

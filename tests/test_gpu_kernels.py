@@ -254,3 +254,24 @@ def test_slot_sum_bit_exact(T, k, N, dtype):
     assert torch.equal(got.cpu(), acc.to(dtype))
     if k > 1:     # and within rounding of the library reduction the reference calls
         _close(got, y.view(T, k, N).float().sum(-2), dtype, scale=float(k) ** 0.5)
+
+
+def test_mfma_rate_probe_launches():
+    """The measurement aid behind bench.py's `mfma_sustained`: launches, reports its flop count, and its sums are
+    what the operands say (zeros stay zero; 16-deep products of values below 2 stay finite)."""
+    import ctypes
+    from scattermoe_amd import _C
+    lib = _C.load()
+    out = torch.full((65536,), float("nan"), device=DEV)
+    flop = ctypes.c_double(0.0)
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    assert lib.smoe_mfma_rate_probe(ctypes.c_void_p(out.data_ptr()), 3, 0, ctypes.byref(flop), st) == 0
+    torch.cuda.synchronize()
+    assert flop.value == 1024 * 3 * 64 * 2.0 * 32 * 32 * 16
+    assert bool((out == 0).all())
+    assert lib.smoe_mfma_rate_probe(None, 3, 1, ctypes.byref(flop), st) == -1                 # SMOE_ERR_NULL
+    assert lib.smoe_mfma_rate_probe(ctypes.c_void_p(out.data_ptr()), 0, 1, ctypes.byref(flop), st) == -5   # SMOE_ERR_RANGE
+    assert lib.smoe_mfma_rate_probe(ctypes.c_void_p(out.data_ptr()), 3, 1, ctypes.byref(flop), st) == 0
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out).all()) and float(out.abs().max()) > 0
+    assert lib.smoe_last_error() == b""
