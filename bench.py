@@ -98,7 +98,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c2")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--cpu-tokens", type=int, default=0, help="token count of the CPU sample (default T/16)")
+    ap.add_argument("--cpu-tokens", type=int, default=0, help="token count of the CPU sample (default T/3)")
     ap.add_argument("--decode", type=int, default=0, metavar="T",
                     help="forward-only latency of one layer at T tokens (decode regime of the workload's expert "
                          "shape); prints its own JSON line with an HBM roofline")
@@ -401,7 +401,7 @@ def main():
         "library_sources": _C.source_hash(),
     }
     if not args.no_cpu:
-        tokens = args.cpu_tokens or max(64, cfg.T // 16)
+        tokens = args.cpu_tokens or max(64, cfg.T // 3)            # c2: about 12 s on 16 cores
         out["cpu_baseline"] = cpu_baseline(cfg, tokens, torch)
     print(json.dumps(out))
 
