@@ -687,6 +687,17 @@ __device__ __forceinline__ void epilogue(const f32x16 (&acc)[TL::FM][TL::FN], T*
 }
 
 // ---- epilogues that go through LDS ------------------------------------------------------------------
+// Two floats rounded to the storage type by one instruction (element-wise casts cost a conversion and a merge per
+// element); same rounding as the scalar cast.  `set_pair` puts the pair into elements 2k, 2k + 1 of a vector.
+template <typename T, typename V>
+__device__ __forceinline__ void set_pair(V& v, int k, float a, float b) {
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  typedef T T2 __attribute__((ext_vector_type(2)));
+  const T2 r = __builtin_convertvector((f32x2_t){a, b}, T2);
+  v[2 * k] = r[0];
+  v[2 * k + 1] = r[1];
+}
+
 // After the main loop the operand buffers are free.  The accumulators (transposed blocks, see `epilogue`) are
 // rounded to the storage type and written to LDS as a row-major BM x BN tile, so that the global traffic of the
 // epilogue can be 16 bytes per lane with a wave covering whole 128-byte lines: 16-byte piece c of row r sits at
@@ -926,12 +937,15 @@ __device__ __forceinline__ void epilogue_glu_fwd_staged(const f32x16 (&acc)[TL::
       const int hc = nh0 + (tc / TL::WTN) * HALF + j % HALF;
       return bias != nullptr && hc < F ? to_f32(bias[(int64_t)(hc + (j >= HALF ? F : 0)) * a.sbn]) : 0.0f;
     }, sbias);
-    const bool gf = (a.act & 1) != 0;
     T* pre = (T*)a.Y;
     T* hid = (T*)a.H;
     // a group's LDS reads are issued back to back ahead of its arithmetic and stores (see epilogue_staged)
     constexpr int GRP = PP >= 8 ? 8 : PP;
     static_assert(PP % GRP == 0, "groups must divide the pieces");
+    // which half holds the gate is the same for the whole launch: one copy of the loop for each case instead of a
+    // select per element (the accumulators are in LDS by now, so the branch has nothing to carry)
+    auto pieces = [&](auto gate_first) {
+    const bool gf = gate_first;       // a constant in the two copies of the one-wave-per-SIMD class
 #pragma unroll
     for (int q0 = 0; q0 < PP; q0 += GRP) {
       T8 v1[GRP], v2[GRP];
@@ -953,8 +967,9 @@ __device__ __forceinline__ void epilogue_glu_fwd_staged(const f32x16 (&acc)[TL::
         const T8 first = v1[g], second = v2[g];
         T8 h;
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-          h[e] = from_f32<T>(glu_h(a.act, to_f32(gf ? first[e] : second[e]), to_f32(gf ? second[e] : first[e])));
+        for (int e = 0; e < 8; e += 2)
+          set_pair<T>(h, e / 2, glu_h(a.act, to_f32(gf ? first[e] : second[e]), to_f32(gf ? second[e] : first[e])),
+                      glu_h(a.act, to_f32(gf ? first[e + 1] : second[e + 1]), to_f32(gf ? second[e + 1] : first[e + 1])));
         const int64_t r = row0 + row;
         if (pre != nullptr) {
           stream_store(first, (T8*)(pre + r * a.sym + n));
@@ -963,6 +978,12 @@ __device__ __forceinline__ void epilogue_glu_fwd_staged(const f32x16 (&acc)[TL::
         stream_store(h, (T8*)(hid + r * a.shm + n));
       }
     }
+    };
+    // (the 8-wave classes, with half the registers per wave, keep one copy and select per element: two copies
+    // there cost 130 spilled registers)
+    if constexpr (!TL::RS) pieces((a.act & 1) != 0);
+    else if ((a.act & 1) != 0) pieces(std::true_type());
+    else pieces(std::false_type());
   }
 }
 
@@ -977,11 +998,13 @@ __device__ __forceinline__ void epilogue_glu_bwd_staged(const f32x16 (&acc)[TL::
   static_assert(PIECES % TL::NT == 0 && (PP == 1 || PP % (2 * GRP) == 0), "pieces must divide evenly");
   stage_accumulators<T, TL>(acc, lds, [](int) { return 0.0f; }, sbias);
   const int F = a.N;
-  const bool gf = (a.act & 1) != 0;
   const T* pre = (const T*)a.aux;
   T* dpre = (T*)a.Y;
   // The saved pre-activation of the next group of pieces is on its way while the current group is worked on (loads of
   // rows and columns outside the tile's valid part are redirected to its first row / column and their results dropped).
+  // One copy of the loop for each position of the gate half (see epilogue_glu_fwd_staged).
+  auto pieces = [&](auto gate_first) {
+  const bool gf = gate_first;       // a constant in the two copies of the one-wave-per-SIMD class
   T8 p1[2][GRP], p2[2][GRP];
   auto fetch = [&](auto buf, int q0) {
 #pragma unroll
@@ -1006,15 +1029,15 @@ __device__ __forceinline__ void epilogue_glu_bwd_staged(const f32x16 (&acc)[TL::
       const int row = p / CPR, n = n0 + (p % CPR) * 8;
       T8 o1, o2;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const T v1 = p1[decltype(buf)::value][u][e], v2 = p2[decltype(buf)::value][u][e];
-        const float dv = to_f32(dh[u][e]);
-        const float lin = to_f32(gf ? v2 : v1), gat = to_f32(gf ? v1 : v2);
-        float f_lin, f_gat;
-        glu_grad(a.act, dv, gat, lin, f_lin, f_gat);
-        const T d_lin = from_f32<T>(f_lin), d_gat = from_f32<T>(f_gat);
-        o1[e] = gf ? d_gat : d_lin;
-        o2[e] = gf ? d_lin : d_gat;
+      for (int e = 0; e < 8; e += 2) {
+        float f_lin[2], f_gat[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const T v1 = p1[decltype(buf)::value][u][e + h], v2 = p2[decltype(buf)::value][u][e + h];
+          glu_grad(a.act, to_f32(dh[u][e + h]), to_f32(gf ? v1 : v2), to_f32(gf ? v2 : v1), f_lin[h], f_gat[h]);
+        }
+        set_pair<T>(o1, e / 2, gf ? f_gat[0] : f_lin[0], gf ? f_gat[1] : f_lin[1]);
+        set_pair<T>(o2, e / 2, gf ? f_lin[0] : f_gat[0], gf ? f_lin[1] : f_gat[1]);
       }
       if (row < rows && n < F) {
         T* dst = dpre + (int64_t)(row0 + row) * a.sym + n;
@@ -1033,6 +1056,10 @@ __device__ __forceinline__ void epilogue_glu_bwd_staged(const f32x16 (&acc)[TL::
       work(std::integral_constant<int, 1>(), q0 + GRP);
     }
   }
+  };
+  if constexpr (!TL::RS) pieces((a.act & 1) != 0);
+  else if ((a.act & 1) != 0) pieces(std::true_type());
+  else pieces(std::false_type());
 }
 
 // gpt-oss forward through LDS: the tile holds BN consecutive columns of the pre-activation, i.e. BN/2 (gate, up)
@@ -1071,7 +1098,9 @@ __device__ __forceinline__ void epilogue_oss_fwd_staged(const f32x16 (&acc)[TL::
       const T8 v = vs[g];
       T4 h;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) h[e] = from_f32<T>(oss_h(to_f32(v[2 * e]), to_f32(v[2 * e + 1]), a.alpha, a.limit));
+      for (int e = 0; e < 4; e += 2)
+        set_pair<T>(h, e / 2, oss_h(to_f32(v[2 * e]), to_f32(v[2 * e + 1]), a.alpha, a.limit),
+                    oss_h(to_f32(v[2 * e + 2]), to_f32(v[2 * e + 3]), a.alpha, a.limit));
       const int64_t r = row0 + row;
       if (pre != nullptr) stream_store(v, (T8*)(pre + r * a.sym + n));
       stream_store(h, (T4*)(hid + r * a.shm + n / 2));
@@ -1121,11 +1150,9 @@ __device__ __forceinline__ void epilogue_oss_bwd_staged(const f32x16 (&acc)[TL::
       for (int e = 0; e < 4; ++e) {
         float dg, du;
         oss_grad(to_f32(v1[2 * e]), to_f32(v1[2 * e + 1]), to_f32(dh[u][e]), a.alpha, a.limit, dg, du);
-        o1[2 * e] = from_f32<T>(dg);
-        o1[2 * e + 1] = from_f32<T>(du);
+        set_pair<T>(o1, e, dg, du);
         oss_grad(to_f32(v2[2 * e]), to_f32(v2[2 * e + 1]), to_f32(dh[u][4 + e]), a.alpha, a.limit, dg, du);
-        o2[2 * e] = from_f32<T>(dg);
-        o2[2 * e + 1] = from_f32<T>(du);
+        set_pair<T>(o2, e, dg, du);
       }
       if (row < rows && n < F) {
         T* dst = dpre + (int64_t)(row0 + row) * a.sym + 2 * n;
