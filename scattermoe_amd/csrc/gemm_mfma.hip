@@ -1047,7 +1047,8 @@ __device__ __forceinline__ void epilogue_glu_bwd_staged(const f32x16 (&acc)[TL::
     }
   };
   fetch(std::integral_constant<int, 0>(), 0);
-#pragma unroll 1
+  // two trips per pass: at the head of a loop the compiler waits for every outstanding load and store
+#pragma unroll 2
   for (int q0 = 0; q0 < PP; q0 += 2 * GRP) {
     if constexpr (PP > 1) fetch(std::integral_constant<int, 1>(), q0 + GRP);
     work(std::integral_constant<int, 0>(), q0);
@@ -1162,7 +1163,8 @@ __device__ __forceinline__ void epilogue_oss_bwd_staged(const f32x16 (&acc)[TL::
     }
   };
   fetch(std::integral_constant<int, 0>(), 0);
-#pragma unroll 1
+  // two trips per pass: at the head of a loop the compiler waits for every outstanding load and store
+#pragma unroll 2
   for (int q0 = 0; q0 < PP; q0 += 2 * GRP) {
     if constexpr (PP > 1) fetch(std::integral_constant<int, 1>(), q0 + GRP);
     work(std::integral_constant<int, 0>(), q0);
