@@ -129,6 +129,19 @@ int smoe_group(const void* A, int64_t sam, int64_t sak, const void* coeff,
                int64_t L, int64_t K, int fan_out, int dtype, void* stream);
 
 /*
+ * smoe_group for an index vector that is a permutation of [0, L), which is what smoe_route produces: the same Y, the
+ * same bits, but every row of A is read once instead of fan_out times (the walk goes by source row and writes its
+ * fan_out scaled copies through the inverse permutation, which a first launch builds in `inverse_workspace`, L
+ * int32 of device memory).  For the `group(grad_out, sorted_scattered_idxs, coeff=gates, fan_out=k)` of
+ * ParallelLinear.backward (scattermoe/parallel_experts.py:88-93).  Rows of Y whose index entry is shared with
+ * another row or lies outside [0, L) are left unwritten - use smoe_group for such vectors.  Returns
+ * SMOE_ERR_UNSUPPORTED (nothing launched) unless rows are contiguous and 16-byte aligned and fan_out <= 64.
+ */
+int smoe_group_by_source(const void* A, int64_t sam, int64_t sak, const void* coeff, void* Y, int64_t sym,
+                         int64_t syk, const int64_t* idx, int32_t* inverse_workspace, int64_t L, int64_t K,
+                         int fan_out, int dtype, void* stream);
+
+/*
  * Per-expert weight / bias gradient over contiguous expert-sorted row ranges.
  * Replaces scattermoe/kernels/ops.py:191-239 (group_bwd_W / op scattermoe::groupXtY), kernels
  * ops.py:242-318, 321-366.

@@ -34,6 +34,7 @@ _SIGNATURES = {
     "smoe_scatter2scatter": (_int, [_p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64,
                                     _p, _p, _p, _i64, _i64, _i64, _int, _int, _int, _int, _int, _p]),
     "smoe_group": (_int, [_p, _i64, _i64, _p, _p, _i64, _i64, _p, _i64, _i64, _int, _int, _p]),
+    "smoe_group_by_source": (_int, [_p, _i64, _i64, _p, _p, _i64, _i64, _p, _p, _i64, _i64, _int, _int, _p]),
     "smoe_groupXtY": (_int, [_p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _i64,
                              _p, _i64, _i64, _i64, _int, _int, _p]),
     "smoe_groupXtY_gathered": (_int, [_p, _i64, _i64, _p, _i64, _i64, _p, _int, _p, _i64, _i64, _i64, _p, _i64, _i64,

@@ -195,6 +195,19 @@ int smoe_group(const void* A, int64_t sam, int64_t sak, const void* coeff, void*
   return launch_group(a, dtype, (hipStream_t)stream);
 }
 
+int smoe_group_by_source(const void* A, int64_t sam, int64_t sak, const void* coeff, void* Y, int64_t sym,
+                         int64_t syk, const int64_t* idx, int32_t* inverse_workspace, int64_t L, int64_t K,
+                         int fan_out, int dtype, void* stream) {
+  g_err[0] = 0;
+  if (!dtype_ok(dtype)) { set_error("smoe_group_by_source: unknown dtype %d", dtype); return SMOE_ERR_DTYPE; }
+  if (L < 0 || K < 0 || fan_out <= 0) { set_error("smoe_group_by_source: bad sizes"); return SMOE_ERR_SHAPE; }
+  if (L > 0x7fffffffLL || K > 0x7fffffffLL) { set_error("smoe_group_by_source: size beyond int32"); return SMOE_ERR_RANGE; }
+  if (L == 0 || K == 0) return 0;
+  if (!A || !Y || !idx || !inverse_workspace) { set_error("smoe_group_by_source: NULL pointer"); return SMOE_ERR_NULL; }
+  GroupArgs a{A, sam, sak, coeff, Y, sym, syk, idx, (int)L, (int)K, fan_out};
+  return launch_group_by_source(a, (int*)inverse_workspace, dtype, (hipStream_t)stream);
+}
+
 int smoe_groupXtY(const void* DY, int64_t sdym, int64_t sdyn, const void* X, int64_t sxm, int64_t sxk,
                   void* DW, int64_t sdwe, int64_t sdwk, int64_t sdwn, void* Db, int64_t sdbe, int64_t sdbn,
                   const int64_t* off, int64_t L, int64_t K, int64_t N, int E, int dtype, void* stream) {

@@ -263,6 +263,7 @@ int launch_route_static(const void* expert_idxs, int idx_dtype, int64_t L, int E
                         int64_t* idx_out, int64_t* off_out, hipStream_t st);
 int route_static_init();
 int launch_offsets_from_sorted(const int64_t* eid, int64_t L, int E, int64_t* off, hipStream_t st);
+int launch_group_by_source(const GroupArgs& a, int* inv, int dtype, hipStream_t st);
 int launch_mfma_rate_probe(float* out, int iters, int random_operands, double* flop, hipStream_t st);
 
 }  // namespace smoe

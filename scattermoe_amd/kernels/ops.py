@@ -75,6 +75,21 @@ class HipBackend:
         _C.check(rc, "smoe_group")
 
     @staticmethod
+    def group_by_source(A, coeff, Y, idx, inverse, fan_out):
+        """True if launched; False if the library does not take these operands (the caller then uses `group`)."""
+        _C.require_gpu(A, "group")
+        lib = _C.load()
+        with _C.on_device(A.device):
+            rc = lib.smoe_group_by_source(_C.ptr(A), A.stride(0), A.stride(1), _C.ptr(coeff),
+                                          _C.ptr(Y), Y.stride(0), Y.stride(1), _C.ptr(idx), _C.ptr(inverse),
+                                          idx.numel(), A.size(1), fan_out, _C.float_code(A.dtype),
+                                          _C.stream_ptr(A.device))
+        if rc == _C.ERR_UNSUPPORTED:
+            return False
+        _C.check(rc, "smoe_group_by_source")
+        return True
+
+    @staticmethod
     def xty(DY, X, DW, Db, off, E):
         _C.require_gpu(DY, "group_bwd_W")
         lib = _C.load()
@@ -497,10 +512,12 @@ def groupXtY_compileable(E: int, DW: torch.Tensor, Db: Optional[torch.Tensor],
 # ------------------------------------------------------------------------------------------------
 # group
 # ------------------------------------------------------------------------------------------------
-def group(A, sorted_expert_idxs, coeff=None, fan_out=1, out=None):
+def group(A, sorted_expert_idxs, coeff=None, fan_out=1, out=None, permutation=False):
     """Y[n] = A[idx[n] // fan_out] * coeff[idx[n]]  (reference ops.py:377-386).
 
     As in the reference the second argument is, despite its name, the sorted *scattered* index vector.
+    `permutation=True` (not in the reference) says that it is a permutation of range(N), as the routing's is: with
+    fan_out > 1 the rows of A are then read once each instead of fan_out times; same result.
     """
     N, K = sorted_expert_idxs.size(0), A.size(1)
     assert A.size(0) * fan_out == N
@@ -508,18 +525,23 @@ def group(A, sorted_expert_idxs, coeff=None, fan_out=1, out=None):
     if torch.compiler.is_compiling():
         group_compileable(A, K, N, Y, coeff, coeff is not None, fan_out, sorted_expert_idxs)
     else:
-        _group_launch(A, Y, coeff, fan_out, sorted_expert_idxs)
+        _group_launch(A, Y, coeff, fan_out, sorted_expert_idxs, permutation)
         _wrote_into(out)
     return Y
 
 
-def _group_launch(A, Y, coeff, fan_out, idx):
+def _group_launch(A, Y, coeff, fan_out, idx, permutation=False):
     assert Y.size(0) == idx.size(0) and Y.size(1) == A.size(1)
     _same_dtype("group", A, Y)
     if coeff is not None:
         assert coeff.numel() == idx.size(0)
         coeff = coeff.reshape(-1).to(A.dtype).contiguous()
-    _backend.group(A, coeff, Y, _as_i64(idx).contiguous(), fan_out)
+    idx = _as_i64(idx).contiguous()
+    if permutation and fan_out > 1 and A.is_cuda and hasattr(_backend, "group_by_source"):
+        inverse = torch.empty(idx.numel(), dtype=torch.int32, device=A.device)
+        if _backend.group_by_source(A, coeff, Y, idx, inverse, fan_out):
+            return
+    _backend.group(A, coeff, Y, idx, fan_out)
 
 
 @torch.library.custom_op("scattermoe::group", mutates_args={"Y"})

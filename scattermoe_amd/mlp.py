@@ -61,7 +61,7 @@ class _GatedMLP(torch.autograd.Function):
             grad_out = grad_out.contiguous()
         d_gates = ops.gate_grad(kept, grad_out) if need_g else None
         # dY of layer 2 in expert-sorted order, scaled by each row's gate; reuses the expert-output buffer
-        dy = ops.group(grad_out, idx, coeff=gates.reshape(-1).to(grad_out.dtype), fan_out=k,
+        dy = ops.group(grad_out, idx, coeff=gates.reshape(-1).to(grad_out.dtype), fan_out=k, permutation=True,
                        out=kept.view(-1, kept.size(-1)))
         d_w2 = d_b2 = None
         if need_w2 or need_b2:

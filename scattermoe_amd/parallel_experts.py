@@ -90,7 +90,7 @@ class ParallelLinear(torch.autograd.Function):
         if grouped_out:
             dy = grad_out
         else:
-            dy = ops.group(grad_out, idx, coeff=coeff, fan_out=coeff_fan, out=dy_buf)
+            dy = ops.group(grad_out, idx, coeff=coeff, fan_out=coeff_fan, out=dy_buf, permutation=True)
 
         d_w = d_b = None
         if need_w or need_b:

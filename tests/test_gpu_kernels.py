@@ -152,6 +152,57 @@ def test_group_bit_exact(T, k, K, with_coeff, dtype):
     assert torch.equal(got2.cpu(), oracle.group_ref(sub[:, 3:K + 3], idx, None, k))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,k,K", [(1, 2, 64), (300, 8, 2048), (777, 4, 2880), (64, 64, 520), (200, 2, 4096 + 64),
+                                   (50, 3, 100)])
+def test_group_walked_by_source_row(T, k, K, dtype):
+    """`permutation=True` reads every source row once and writes its k scaled copies through the inverse
+    permutation: the oracle's values and the same bits as the gather, for rows longer than one pass of a wave
+    (more than 2048 16-bit columns), row lengths that are no multiple of a pass, k up to a whole wave, and row
+    lengths the 16-byte path does not take (the call then falls back to the gather)."""
+    g = torch.Generator().manual_seed(T * k + K)
+    experts = torch.stack([torch.randperm(max(k, 8), generator=g)[:k] for _ in range(T)])
+    _, idx, _ = oracle.route_ref(experts, max(k, 8))
+    A = torch.randn(T, K, generator=g).to(dtype)
+    coeff = torch.rand(T * k, generator=g).to(dtype)
+    want = oracle.group_ref(A, idx, coeff, fan_out=k)
+    out = torch.full((T * k + 2, K), float("nan"), dtype=dtype, device=DEV)      # a guard row on either side
+    got = ops.group(A.to(DEV), idx.to(DEV), coeff=coeff.to(DEV), fan_out=k, out=out[1:-1], permutation=True)
+    assert torch.equal(got.cpu(), want)
+    assert bool(torch.isnan(out[0]).all()) and bool(torch.isnan(out[-1]).all())
+    assert torch.equal(got, ops.group(A.to(DEV), idx.to(DEV), coeff=coeff.to(DEV), fan_out=k))
+
+
+def test_group_walked_by_source_row_skips_what_is_not_a_permutation():
+    """An index vector with a repeated and an out-of-range entry, and a workspace full of stale values: rows whose
+    index entry is theirs alone get the gather's values, and nothing is written outside Y."""
+    import ctypes
+    from scattermoe_amd import _C
+    T, k, K = 40, 4, 256
+    L = T * k
+    g = torch.Generator().manual_seed(5)
+    idx = torch.randperm(L, generator=g)
+    idx[7] = idx[3]                       # slot idx[3] claimed twice, the slot that row 7 had by nobody
+    idx[11] = L + 5                       # out of range
+    A = torch.randn(T, K, generator=g).bfloat16().to(DEV)
+    coeff = torch.rand(L, generator=g).bfloat16().to(DEV)
+    Y = torch.full((L + 2, K), float("nan"), dtype=torch.bfloat16, device=DEV)
+    inv = torch.randint(-2 ** 31, 2 ** 31 - 1, (L,), generator=g, dtype=torch.int64).to(torch.int32).to(DEV)
+    lib = _C.load()
+    idx_d = idx.to(DEV)
+    rc = lib.smoe_group_by_source(_C.ptr(A), A.stride(0), 1, _C.ptr(coeff), _C.ptr(Y[1:]), K, 1, _C.ptr(idx_d),
+                                  _C.ptr(inv), L, K, k, _C.float_code(A.dtype), _C.stream_ptr(A.device))
+    assert rc == 0
+    torch.cuda.synchronize()
+    got = Y[1:-1].cpu()
+    sure = [r for r in range(L) if r not in (3, 7, 11)]
+    want = (A.cpu().float()[idx[sure] // k] * coeff.cpu().float()[idx[sure]].unsqueeze(1)).bfloat16()
+    assert torch.equal(got[sure], want)
+    assert bool(torch.isnan(got[11]).all())                          # its slot does not exist
+    assert bool(torch.isnan(got[3]).all()) != bool(torch.isnan(got[7]).all())      # one of the two claimants wins
+    assert bool(torch.isnan(Y[0]).all()) and bool(torch.isnan(Y[-1]).all())
+
+
 # ---------------------------------------------------------------------------------------------------
 # groupXtY
 # ---------------------------------------------------------------------------------------------------
