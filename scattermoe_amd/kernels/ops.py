@@ -488,7 +488,7 @@ def group_bwd_W(DY, X, expert_offsets, E, has_bias=False, like=None, gather=None
             if _backend.xty_gathered(DY, X, _as_i64(idx).contiguous(), fan_out, DW, Db,
                                      _as_i64(expert_offsets).contiguous(), E):
                 return DW, Db
-        X = group(X, idx, fan_out=fan_out)
+        X = group(X, idx, fan_out=fan_out, permutation=True)   # `gather` is the routing's index vector
     if torch.compiler.is_compiling():
         groupXtY_compileable(E, DW, Db, DY, X, expert_offsets)
     else:
