@@ -39,8 +39,33 @@ __global__ __launch_bounds__(256) void combine_kernel(const T* __restrict__ Y, i
       float acc[P::n];
 #pragma unroll
       for (int q = 0; q < P::n; ++q) acc[q] = 0.0f;
-      for (int j = 0; j < k; ++j) {
-        const float g = G ? to_f32(G[t * sgt + j * sgk]) : 1.0f;      // no gates: plain sum over the k slots
+      // four slots' loads in flight at a time; the sum runs over the slots in order either way
+      int j = 0;
+      for (; j + 4 <= k; j += 4) {
+        P x[4];
+        float g[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          x[u] = stream_load16<P>(y0 + (j + u) * sy + (int64_t)c * P::n);
+          g[u] = G ? to_f32(G[t * sgt + (j + u) * sgk]) : 1.0f;       // no gates: plain sum over the k slots
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+          for (int q = 0; q < P::n; ++q) acc[q] = fmaf(g[u], to_f32(x[u].v[q]), acc[q]);
+      }
+      if (j + 2 <= k) {
+        const P x0 = stream_load16<P>(y0 + j * sy + (int64_t)c * P::n);
+        const P x1 = stream_load16<P>(y0 + (j + 1) * sy + (int64_t)c * P::n);
+        const float g0 = G ? to_f32(G[t * sgt + j * sgk]) : 1.0f, g1 = G ? to_f32(G[t * sgt + (j + 1) * sgk]) : 1.0f;
+#pragma unroll
+        for (int q = 0; q < P::n; ++q) acc[q] = fmaf(g0, to_f32(x0.v[q]), acc[q]);
+#pragma unroll
+        for (int q = 0; q < P::n; ++q) acc[q] = fmaf(g1, to_f32(x1.v[q]), acc[q]);
+        j += 2;
+      }
+      if (j < k) {
+        const float g = G ? to_f32(G[t * sgt + j * sgk]) : 1.0f;
         const P x = stream_load16<P>(y0 + j * sy + (int64_t)c * P::n);
 #pragma unroll
         for (int q = 0; q < P::n; ++q) acc[q] = fmaf(g, to_f32(x.v[q]), acc[q]);
