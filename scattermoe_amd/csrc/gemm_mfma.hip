@@ -1286,17 +1286,20 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
   // first output column of the tile; the fused forward GLU tile holds BN/2 columns of each half
   const int n0 = a.glu == 1 ? n_tile * (TL::BN / 2) : n_tile * TL::BN;
 
-  for (int m = threadIdx.x; m < TL::BM; m += TL::NT) {
-    const int mm = m < rows ? m : rows - 1;               // tail rows re-read the last valid row
-    const int64_t n = row0 + mm;
-    int64_t src = n, dst = n;
-    if (!a.x_grouped || !a.y_grouped) {
-      const int64_t i = a.idx[n];
-      if (!a.x_grouped) src = i / a.fan_out;
-      if (!a.y_grouped) dst = i;
+  // Row tables, one tile row per thread.  The main loop needs only the source rows; where the output rows go is
+  // stored after it, so that a launch whose input is grouped and whose output is not (layer-2 forward, layer-1
+  // input gradient) does not wait for the index vector before its first operand loads.
+  static_assert(TL::BM <= TL::NT, "one row of the tables per thread");
+  int64_t slot = 0;                                         // idx[n] where it is needed, else unused
+  int64_t own_row = 0;
+  {
+    const int m = threadIdx.x;
+    if (m < TL::BM) {
+      const int mm = m < rows ? m : rows - 1;               // tail rows re-read the last valid row
+      own_row = row0 + mm;
+      if (!a.x_grouped || !a.y_grouped) slot = a.idx[own_row];
+      sSrc[m] = a.x_grouped ? (int)own_row : (int)(slot / a.fan_out);
     }
-    sSrc[m] = (int)src;
-    sDst[m] = m < rows ? dst * a.sym : -1;
   }
   __syncthreads();
 
@@ -1345,6 +1348,12 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
   else if constexpr (TL::NS > 2) mainloop_ring<T, TL, AOp, BOp>(A, B, a.K, lds, acc);
   else mainloop<T, TL, AOp, BOp, false>(A, B, a.K, lds, false, acc, rs);
 
+  {
+    asm volatile("" : "+v"(slot), "+v"(own_row));           // not looked at before this point
+    const int m = threadIdx.x;
+    if (m < TL::BM) sDst[m] = m < rows ? (a.y_grouped ? own_row : slot) * a.sym : -1;
+  }
+  __syncthreads();
   const T* bias = a.b ? (const T*)a.b + (int64_t)e * a.sbe : nullptr;
   // 16-byte pieces need every row start 16-byte aligned; otherwise the lane-wise epilogues are used (the
   // one-wave-per-SIMD class is only launched on aligned outputs)
