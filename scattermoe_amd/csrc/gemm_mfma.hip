@@ -885,6 +885,25 @@ __device__ __forceinline__ void epilogue_glu_bwd(const f32x16 (&acc)[TL::FM][TL:
 template <typename V>
 __device__ __forceinline__ void stream_store(const V& v, V* p) { __builtin_nontemporal_store(v, p); }
 
+// 16-byte store through a buffer descriptor: the hardware drops it when `offset` (bytes) lies beyond the descriptor's
+// range, so a piece outside the tile's valid part needs no branch around its store.  That matters where loads are in
+// flight across the stores: stores and loads share one counter, and behind a store that a branch may have skipped
+// the compiler can only wait for everything, the prefetched loads of the next group included.
+template <typename V>
+__device__ __forceinline__ void range_checked_store(const V& v, __amdgpu_buffer_rsrc_t r, unsigned offset) {
+  static_assert(sizeof(V) == 16, "16-byte pieces");
+  typedef unsigned u32x4_st __attribute__((ext_vector_type(4)));
+  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_st, v), r, (int)offset, 0, 2 /* non-temporal */);
+}
+// Descriptor over the valid rows of a tile's output: `row_bytes` per row from `base` on.
+// (Base and range are the same for every lane; saying so keeps the compiler from wrapping each store into a loop
+// over the distinct descriptors of the wave.)
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_rows_rsrc(void* base, int rows, int64_t row_bytes) {
+  const int64_t span = (int64_t)rows * row_bytes;
+  const int range = __builtin_amdgcn_readfirstlane(span < 0xffffffffLL ? (int)(unsigned)span : -1);
+  return __builtin_amdgcn_make_buffer_rsrc((void*)make_uniform((const char*)base), 0, range, 0x00020000);
+}
+
 template <typename T, class TL>
 __device__ __forceinline__ void epilogue_staged(const f32x16 (&acc)[TL::FM][TL::FN], T* __restrict__ out,
                                                 const int64_t* dst, int n0, int ncols, const T* __restrict__ bias,
@@ -1000,6 +1019,7 @@ __device__ __forceinline__ void epilogue_glu_bwd_staged(const f32x16 (&acc)[TL::
   const int F = a.N;
   const T* pre = (const T*)a.aux;
   T* dpre = (T*)a.Y;
+  const __amdgpu_buffer_rsrc_t out_rows = tile_rows_rsrc(dpre + (int64_t)row0 * a.sym, rows, a.sym * 2);
   // The saved pre-activation of the next group of pieces is on its way while the current group is worked on (loads of
   // rows and columns outside the tile's valid part are redirected to its first row / column and their results dropped).
   // One copy of the loop for each position of the gate half (see epilogue_glu_fwd_staged).
@@ -1039,11 +1059,9 @@ __device__ __forceinline__ void epilogue_glu_bwd_staged(const f32x16 (&acc)[TL::
         set_pair<T>(o1, e / 2, gf ? f_gat[0] : f_lin[0], gf ? f_gat[1] : f_lin[1]);
         set_pair<T>(o2, e / 2, gf ? f_lin[0] : f_gat[0], gf ? f_lin[1] : f_gat[1]);
       }
-      if (row < rows && n < F) {
-        T* dst = dpre + (int64_t)(row0 + row) * a.sym + n;
-        stream_store(o1, (T8*)dst);
-        stream_store(o2, (T8*)(dst + F));
-      }
+      const unsigned at = row < rows && n < F ? (unsigned)(((int64_t)row * a.sym + n) * 2) : 0xffffffffu;
+      range_checked_store(o1, out_rows, at);
+      range_checked_store(o2, out_rows, at == 0xffffffffu ? at : at + (unsigned)F * 2);
     }
   };
   fetch(std::integral_constant<int, 0>(), 0);
@@ -1122,6 +1140,7 @@ __device__ __forceinline__ void epilogue_oss_bwd_staged(const f32x16 (&acc)[TL::
   const int F = a.N;
   const T* pre = (const T*)a.aux;
   T* dpre = (T*)a.Y;
+  const __amdgpu_buffer_rsrc_t out_rows = tile_rows_rsrc(dpre + (int64_t)row0 * a.sym, rows, a.sym * 2);
   // next group's saved pre-activation pairs on their way while the current group is worked on (see epilogue_glu_bwd_staged)
   T8 p1[2][GRP], p2[2][GRP];
   auto fetch = [&](auto buf, int q0) {
@@ -1155,11 +1174,9 @@ __device__ __forceinline__ void epilogue_oss_bwd_staged(const f32x16 (&acc)[TL::
         oss_grad(to_f32(v2[2 * e]), to_f32(v2[2 * e + 1]), to_f32(dh[u][4 + e]), a.alpha, a.limit, dg, du);
         set_pair<T>(o2, e, dg, du);
       }
-      if (row < rows && n < F) {
-        T* dst = dpre + (int64_t)(row0 + row) * a.sym + 2 * n;
-        stream_store(o1, (T8*)dst);
-        stream_store(o2, (T8*)(dst + 8));
-      }
+      const unsigned at = row < rows && n < F ? (unsigned)(((int64_t)row * a.sym + 2 * n) * 2) : 0xffffffffu;
+      range_checked_store(o1, out_rows, at);
+      range_checked_store(o2, out_rows, at == 0xffffffffu ? at : at + 16u);
     }
   };
   fetch(std::integral_constant<int, 0>(), 0);
