@@ -1517,6 +1517,8 @@ static int dispatch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
     return SMOE_ERR_UNSUPPORTED;
   if (a.glu == 4 && !((((uintptr_t)a.aux | (uintptr_t)a.Y) & 15) == 0 && ((a.saux | a.sym | a.N) & 7) == 0))
     return SMOE_ERR_UNSUPPORTED;
+  // the backward gated epilogues address a tile's output rows with 32-bit byte offsets from its first row
+  if ((a.glu == 2 || a.glu == 4) && a.sym * 2 * 256 >= 0xffffffffLL) return SMOE_ERR_UNSUPPORTED;
   const int64_t avg = a.L / a.E;
   if (const int m_first = avg >= ROWS256_BELOW ? tail_split(a) : 0) {
     S2SArgs first = a, rest = a;
