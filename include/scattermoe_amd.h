@@ -119,6 +119,28 @@ int smoe_scatter2scatter(const void* X, int64_t sxm, int64_t sxk,
                          int x_grouped, int y_grouped, int dtype, void* stream);
 
 /*
+ * smoe_scatter2scatter with a caller workspace (same reference function, scattermoe/kernels/ops.py:120-183; the
+ * reference has no such argument).  Every expert ends in a partly filled tile of rows; in a product with many rows
+ * per expert, few output columns and a long contraction (Mixtral layer-2 forward and layer-1 input gradient:
+ * 8 experts x 16 tile columns) those tiles are too few to fill the chip and each walks the whole contraction.
+ * With `workspace` of at least smoe_scatter2scatter_workspace_bytes(L, K, N, E, dtype) bytes (16-byte aligned)
+ * their contraction is cut into parts that run side by side; a second small launch adds the float32 partial
+ * sums in a fixed order and writes the rows.  Results are the same on every run, and within float32 rounding
+ * of - not bit-identical to - the product without workspace (the additions are grouped differently).
+ * workspace == NULL or too small: exactly smoe_scatter2scatter.  The workspace is free again when the launches
+ * of the call have run.  smoe_scatter2scatter_workspace_bytes returns 0 for products that would not use one.
+ */
+size_t smoe_scatter2scatter_workspace_bytes(int64_t L, int64_t K, int64_t N, int E, int dtype);
+int smoe_scatter2scatter_ws(const void* X, int64_t sxm, int64_t sxk,
+                            const void* W, int64_t swe, int64_t swk, int64_t swn,
+                            const void* b, int64_t sbe, int64_t sbn,
+                            void* Y, int64_t sym, int64_t syn,
+                            const int64_t* eid, const int64_t* idx, const int64_t* off,
+                            int64_t L, int64_t K, int64_t N, int E, int fan_out,
+                            int x_grouped, int y_grouped, int dtype,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Row gather into expert-sorted order with optional per-row coefficient.
  * Replaces scattermoe/kernels/ops.py:377-410 (group / op scattermoe::group), kernel ops.py:413-457.
  *   Y[n, :] = A[idx[n] / fan_out, :] * (coeff ? coeff[idx[n]] : 1)      n in [0,L)

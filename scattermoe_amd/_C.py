@@ -33,6 +33,9 @@ _SIGNATURES = {
     "smoe_offsets_from_sorted": (_int, [_p, _i64, _int, _p, _p]),
     "smoe_scatter2scatter": (_int, [_p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64,
                                     _p, _p, _p, _i64, _i64, _i64, _int, _int, _int, _int, _int, _p]),
+    "smoe_scatter2scatter_workspace_bytes": (_sz, [_i64, _i64, _i64, _int, _int]),
+    "smoe_scatter2scatter_ws": (_int, [_p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64,
+                                       _p, _p, _p, _i64, _i64, _i64, _int, _int, _int, _int, _int, _p, _sz, _p]),
     "smoe_group": (_int, [_p, _i64, _i64, _p, _p, _i64, _i64, _p, _i64, _i64, _int, _int, _p]),
     "smoe_group_by_source": (_int, [_p, _i64, _i64, _p, _p, _i64, _i64, _p, _p, _i64, _i64, _int, _int, _p]),
     "smoe_groupXtY": (_int, [_p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _i64,

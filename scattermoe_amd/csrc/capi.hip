@@ -86,11 +86,25 @@ int smoe_offsets_from_sorted(const int64_t* eid, int64_t L, int E, int64_t* off_
   return launch_offsets_from_sorted(eid, L, E, off_out, (hipStream_t)stream);
 }
 
+size_t smoe_scatter2scatter_workspace_bytes(int64_t L, int64_t K, int64_t N, int E, int dtype) {
+  if (L <= 0 || K <= 0 || N <= 0 || E <= 0) return 0;
+  return (size_t)s2s_workspace_floats(L, K, N, E, dtype) * sizeof(float);
+}
+
 int smoe_scatter2scatter(const void* X, int64_t sxm, int64_t sxk, const void* W, int64_t swe, int64_t swk,
                          int64_t swn, const void* b, int64_t sbe, int64_t sbn, void* Y, int64_t sym,
                          int64_t syn, const int64_t* eid, const int64_t* idx, const int64_t* off, int64_t L,
                          int64_t K, int64_t N, int E, int fan_out, int x_grouped, int y_grouped, int dtype,
                          void* stream) {
+  return smoe_scatter2scatter_ws(X, sxm, sxk, W, swe, swk, swn, b, sbe, sbn, Y, sym, syn, eid, idx, off, L, K, N, E,
+                                 fan_out, x_grouped, y_grouped, dtype, nullptr, 0, stream);
+}
+
+int smoe_scatter2scatter_ws(const void* X, int64_t sxm, int64_t sxk, const void* W, int64_t swe, int64_t swk,
+                            int64_t swn, const void* b, int64_t sbe, int64_t sbn, void* Y, int64_t sym,
+                            int64_t syn, const int64_t* eid, const int64_t* idx, const int64_t* off, int64_t L,
+                            int64_t K, int64_t N, int E, int fan_out, int x_grouped, int y_grouped, int dtype,
+                            void* workspace, size_t workspace_bytes, void* stream) {
   g_err[0] = 0;
   if (!dtype_ok(dtype)) { set_error("smoe_scatter2scatter: unknown dtype %d", dtype); return SMOE_ERR_DTYPE; }
   if (L < 0 || K < 0 || N < 0 || E <= 0 || fan_out <= 0) { set_error("smoe_scatter2scatter: bad sizes"); return SMOE_ERR_SHAPE; }
@@ -100,6 +114,10 @@ int smoe_scatter2scatter(const void* X, int64_t sxm, int64_t sxk, const void* W,
   (void)eid;  // expert boundaries come from `off`; kept in the signature for parity with the reference call
   S2SArgs a{X, sxm, sxk, W, swe, swk, swn, b, sbe, sbn, Y, sym, syn, eid, idx, off,
             (int)L, (int)K, (int)N, E, fan_out, x_grouped, y_grouped};
+  if (workspace != nullptr && ((uintptr_t)workspace & 15) == 0) {       // optional: without it nothing is split
+    a.partial = (float*)workspace;
+    a.partial_floats = (int64_t)(workspace_bytes / sizeof(float));
+  }
   int rc = 0;
   if (try_s2s_mfma(a, dtype, (hipStream_t)stream, rc)) return rc;
   return launch_s2s_generic(a, dtype, (hipStream_t)stream);
@@ -231,6 +249,10 @@ int smoe_groupXtY_gathered(const void* DY, int64_t sdym, int64_t sdyn, const voi
   if (!dtype_ok(dtype)) { set_error("smoe_groupXtY_gathered: unknown dtype %d", dtype); return SMOE_ERR_DTYPE; }
   if (L < 0 || K < 0 || N < 0 || E <= 0 || fan_out <= 0) { set_error("smoe_groupXtY_gathered: bad sizes"); return SMOE_ERR_SHAPE; }
   if (L > 0x7fffffffLL || K > 0x7fffffffLL || N > 0x7fffffffLL) { set_error("smoe_groupXtY_gathered: size beyond int32"); return SMOE_ERR_RANGE; }
+  if (L % fan_out != 0) { set_error("smoe_groupXtY_gathered: L=%lld is not a multiple of fan_out=%d", (long long)L, fan_out); return SMOE_ERR_SHAPE; }
+  // Only the bf16 / fp16 MFMA kernel reads X through the index vector; the float32 kernels would take X for the
+  // grouped (L, K) matrix and read past the end of the (L / fan_out, K) one.  Nothing is launched.
+  if (dtype == SMOE_F32) { set_error("smoe_groupXtY_gathered: float32 is not gathered; group X and call smoe_groupXtY"); return SMOE_ERR_UNSUPPORTED; }
   if (K == 0 || N == 0) return 0;
   if (!DW || !off || (L > 0 && (!DY || !X || !idx))) { set_error("smoe_groupXtY_gathered: NULL pointer"); return SMOE_ERR_NULL; }
   XtYArgs a{DY, sdym, sdyn, X, sxm, sxk, DW, sdwe, sdwk, sdwn, Db, sdbe, sdbn, off, (int)L, (int)K, (int)N, E};

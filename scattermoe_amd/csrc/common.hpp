@@ -191,6 +191,12 @@ struct S2SArgs {
   // Products whose experts end in a partly filled tile (MFMA path only).  1: this launch leaves out every expert's
   // last tile when it holds at most 128 rows; 2: this launch takes exactly those rows, one tile row per expert.
   int tail_mode = 0;
+  // tail_mode 2 only: the contraction of every tile is cut into `ksplit` equal parts, one workgroup each, which
+  // leave their float32 accumulators in `partial` (see splitk_floats); a second launch adds the parts up in a
+  // fixed order and writes the output rows.  `partial` / `partial_floats`: the caller's workspace, may be NULL / 0.
+  int ksplit = 1, k_part = 0;           // k_part = K / ksplit
+  float* partial = nullptr;
+  int64_t partial_floats = 0;
 };
 
 struct XtYArgs {
@@ -235,6 +241,9 @@ int launch_xty_generic(const XtYArgs& a, int dtype, hipStream_t st);
 int launch_group(const GroupArgs& a, int dtype, hipStream_t st);
 // MFMA paths return 1 if they took the call, 0 if the shape/layout is not theirs, <0 / >1 never.
 bool try_s2s_mfma(const S2SArgs& a, int dtype, hipStream_t st, int& rc);
+// float32 values of workspace with which a plain bf16 / fp16 product of these sizes can split the contraction of
+// its experts' last, sparsely filled tiles (0: the product would not use one)
+int64_t s2s_workspace_floats(int64_t L, int64_t K, int64_t N, int E, int dtype);
 bool try_s2s_f32(const S2SArgs& a, hipStream_t st, int& rc);     // float32 MFMA paths (csrc/gemm_f32.hip)
 bool try_xty_f32(const XtYArgs& a, hipStream_t st, int& rc);
 bool try_s2s_rowdot(const S2SArgs& a, int dtype, hipStream_t st, int& rc);   // few-row launches; after try_s2s_mfma's checks

@@ -1289,6 +1289,15 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
   __shared__ int sSrc[TL::BM];
   __shared__ __attribute__((aligned(16))) float sBias[TL::RS ? TL::BN : 4];
 
+  // Contraction parts (the class of the experts' last tiles only): the grid is `ksplit` copies of the raster, copy
+  // c multiplies the c-th part of the contraction (a raster is a multiple of 8 workgroups, so the XCD of a workgroup
+  // is still its first index modulo 8)
+  constexpr bool CAN_SPLIT = TL::BM == 128 && TL::BN == 256 && TL::NS == 3;
+  // (the parts are the grid's second dimension; no division here: the compiler would do it in the vector unit and
+  // everything derived from it, loop counters and LDS addresses included, would leave the scalar registers)
+  const int part = CAN_SPLIT ? (int)blockIdx.y : 0;
+  const int klen = CAN_SPLIT && a.ksplit > 1 ? a.k_part : a.K;
+  const int k_first = part * klen;
   int m_tile, n_tile, m_loc, n_loc;
   if (!rast.map(blockIdx.x, m_tile, n_tile, m_loc, n_loc)) return;
   int e, row0, rows;
@@ -1326,11 +1335,11 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
   // be of any size), gathered ones relative to the start of the token matrix.
   const int64_t sxm = a.sxm;
   const int src0 = a.x_grouped ? row0 : 0;
-  const char* Xb = (const char*)a.X + (int64_t)src0 * sxm * 2;
+  const char* Xb = (const char*)a.X + ((int64_t)src0 * sxm + k_first) * 2;
   A.init(Xb, [&](int row) { return (int64_t)(sSrc[row] - src0) * sxm * 2; });
   BOp B;
   B.rot = TL::RS ? 0 : (m_loc * BOp::R / Raster::SM) % BOp::R;      // the column panel has SM sharers
-  const char* Wb = (const char*)a.W + (int64_t)e * a.swe * 2;
+  const char* Wb = (const char*)a.W + ((int64_t)e * a.swe + (int64_t)k_first * (B_TR ? a.swk : 1)) * 2;
   if (a.glu == 1) {
     // tile column tc -> weight column: wave block tc / WTN, first half of the block from [0, F), second from [F, 2F)
     const int F = a.N;
@@ -1362,8 +1371,27 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
   if constexpr (TL::RS) mainloop_rs<T, TL, AOp, BOp>(A, B, a.K, lds, acc);
-  else if constexpr (TL::NS > 2) mainloop_ring<T, TL, AOp, BOp>(A, B, a.K, lds, acc);
+  else if constexpr (TL::NS > 2) mainloop_ring<T, TL, AOp, BOp>(A, B, klen, lds, acc);
   else mainloop<T, TL, AOp, BOp, false>(A, B, a.K, lds, false, acc, rs);
+
+  if constexpr (CAN_SPLIT) {
+    if (a.ksplit > 1) {
+      // This part's accumulators as they lie in the registers, 16 bytes per lane and store (whole 1 KB runs per
+      // wave); splitk_reduce_kernel knows which output element each of them belongs to.
+      typedef float f32x4_t __attribute__((ext_vector_type(4)));
+      f32x4_t* P = (f32x4_t*)a.partial +
+                   (((int64_t)e * rast.n_tiles + n_tile) * a.ksplit + part) * (TL::FM * TL::FN * 4 * TL::NT);
+#pragma unroll
+      for (int i = 0; i < TL::FM; ++i)
+#pragma unroll
+        for (int j = 0; j < TL::FN; ++j)
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+            P[((i * TL::FN + j) * 4 + g) * TL::NT + threadIdx.x] =
+                f32x4_t{acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+      return;
+    }
+  }
 
   {
     asm volatile("" : "+v"(slot), "+v"(own_row));           // not looked at before this point
@@ -1399,6 +1427,56 @@ __global__ __launch_bounds__(TL::NT) void s2s_mfma_kernel(S2SArgs a, Raster rast
   }
 }
 
+// Second half of a product whose last tiles were multiplied in contraction parts: one workgroup per (expert, tile
+// column) with the thread layout of the 128 x 256 class, so that thread t finds the accumulators that thread t of
+// every part left behind.  The parts are added in ascending order (the same result on every run), then bias,
+// rounding and the scatter of the rows as in the plain epilogue.
+template <typename T>
+__global__ __launch_bounds__(512) void splitk_reduce_kernel(S2SArgs a, int n_tiles) {
+  typedef Tile<128, 256, 2, 4, 3> TL;
+  typedef float f32x4_t __attribute__((ext_vector_type(4)));
+  typedef T T4 __attribute__((ext_vector_type(4)));
+  const int e = blockIdx.y, n_tile = blockIdx.x;
+  int row0, rows;
+  if (!find_remainder<256>(a.off, a.E, e, TL::BM, row0, rows)) return;
+  const int wave = threadIdx.x >> 6, l = lane_id();
+  const int wm = wave / TL::WN, wn = wave % TL::WN;
+  const f32x4_t* P = (const f32x4_t*)a.partial + ((int64_t)e * n_tiles + n_tile) * a.ksplit * (TL::FM * TL::FN * 4 * TL::NT);
+  const T* bias = a.b ? (const T*)a.b + (int64_t)e * a.sbe : nullptr;
+  T* out = (T*)a.Y;
+  const bool base_ok = ((uintptr_t)out & 7) == 0;
+#pragma unroll
+  for (int i = 0; i < TL::FM; ++i) {
+    const int m = wm * TL::WTM + i * 32 + (l & 31);
+    if (m >= rows) continue;
+    const int64_t row = row0 + m;
+    const int64_t d = (a.y_grouped ? row : a.idx[row]) * a.sym;
+#pragma unroll
+    for (int j = 0; j < TL::FN; ++j) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int n = n_tile * TL::BN + wn * TL::WTN + j * 32 + g * 8 + (l >> 5) * 4;
+        if (n >= a.N) continue;
+        const int slot = ((i * TL::FN + j) * 4 + g) * TL::NT + threadIdx.x;
+        f32x4_t v = P[slot];
+        for (int c = 1; c < a.ksplit; ++c) v += P[(int64_t)c * (TL::FM * TL::FN * 4 * TL::NT) + slot];
+        if (bias != nullptr) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            if (n + q < a.N) v[q] += to_f32(bias[(int64_t)(n + q) * a.sbn]);
+        }
+        if (base_ok && n + 3 < a.N && ((d + n) & 3) == 0) {
+          *(T4*)(out + d + n) = T4{from_f32<T>(v[0]), from_f32<T>(v[1]), from_f32<T>(v[2]), from_f32<T>(v[3])};
+        } else {
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            if (n + q < a.N) out[d + n + q] = from_f32<T>(v[q]);
+        }
+      }
+    }
+  }
+}
+
 template <typename T, class TL>
 static int launch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
   const int bn = a.glu == 1 ? TL::BN / 2 : TL::BN;     // output columns per tile
@@ -1409,14 +1487,15 @@ static int launch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
   const bool striped = TL::NS > 2 || a.L / a.E < STRIPE_BELOW;
   const Raster r = striped ? make_striped(m_tiles, n_tiles, GM_RING) : make_raster(m_tiles, n_tiles, GM_S2S);
   const int64_t grid = r.grid();
+  const unsigned parts = a.ksplit > 1 ? (unsigned)a.ksplit : 1u;
   if (grid > 0x7fffffffLL || m_tiles > 0x7fffffffLL) { set_error("smoe_scatter2scatter: grid too large"); return SMOE_ERR_RANGE; }
   if constexpr (TL::BN % 128 == 0) {
     if (b_tr) {
-      hipLaunchKernelGGL((s2s_mfma_kernel<T, TL, true>), dim3((unsigned)grid), dim3(TL::NT), 0, st, a, r);
+      hipLaunchKernelGGL((s2s_mfma_kernel<T, TL, true>), dim3((unsigned)grid, parts), dim3(TL::NT), 0, st, a, r);
       return launch_status("s2s_mfma_kernel");
     }
   }
-  hipLaunchKernelGGL((s2s_mfma_kernel<T, TL, false>), dim3((unsigned)grid), dim3(TL::NT), 0, st, a, r);
+  hipLaunchKernelGGL((s2s_mfma_kernel<T, TL, false>), dim3((unsigned)grid, parts), dim3(TL::NT), 0, st, a, r);
   return launch_status("s2s_mfma_kernel");
 }
 
@@ -1428,13 +1507,19 @@ static int launch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
 // anywhere between 800 and 3136 tokens.
 static constexpr int NUM_CU = 256;
 static constexpr double HALF_WIDTH_COST = 0.58;
-// expected number of 256-row tiles, rounded
-static double expected_row_tiles(int64_t L, int E) {
+// expected number of 256-row tiles, rounded; `skip_small`: without the experts' last tiles of at most that many rows
+static double expected_row_tiles(int64_t L, int E, int skip_small = 0) {
   const double avg = (double)L / E, sd = sqrt(avg * (1.0 - 1.0 / E)) + 1e-9;
+  auto above = [&](double x) { return 0.5 * erfc((x - avg) / (sd * 1.41421356)); };      // P(rows > x)
   // expected ceil(rows / 256) = 1 + sum_j P(rows > 256 j); the terms more than 6 sd below the mean are 1
   const int j_lo = std::max(1, (int)((avg - 6 * sd) / 256.0));
   double per_expert = j_lo;
-  for (int j = j_lo; j * 256.0 < avg + 6 * sd; ++j) per_expert += 0.5 * erfc((j * 256.0 - avg) / (sd * 1.41421356));
+  for (int j = j_lo; j * 256.0 < avg + 6 * sd; ++j) per_expert += above(j * 256.0);
+  if (skip_small > 0) {
+    // minus P(rows mod 256 in [1, skip_small])
+    for (int j = std::max(0, j_lo - 1); j * 256.0 < avg + 6 * sd; ++j)
+      per_expert -= above(j * 256.0 + 0.5) - above(j * 256.0 + skip_small + 0.5);
+  }
   return nearbyint(per_expert * E);
 }
 static bool half_width_wins(const S2SArgs& a) {
@@ -1459,12 +1544,14 @@ static int tail_split(const S2SArgs& a) {
   const int64_t n_full = (a.N + 255) / 256;
   const int64_t upper = max_tiles(a.L, a.E, 256);
   if (upper * n_full > 26 * NUM_CU) return 0;
-  const double m = expected_row_tiles(a.L, a.E);
+  const double m = expected_row_tiles(a.L, a.E, a.tail_mode == 1 ? REMAINDER_ROWS : 0);
   const int64_t whole = (int64_t)(m * n_full) / NUM_CU;           // whole rounds
   if (whole < 2) return 0;
   const int64_t m_first = whole * NUM_CU / n_full;                // tile rows that fit the whole rounds
   const int64_t rest = ((int64_t)m - m_first) * n_full;           // expected 256 x 256 tiles of the remainder
-  if (m_first <= 0 || rest <= 0 || upper <= m_first || rest > NUM_CU / 2 + 8) return 0;
+  // (no remainder expected: the second launch still stands by for a tile row more than expected, which would
+  // otherwise cost the first launch a whole round; its workgroups exit at once when there is none)
+  if (m_first <= 0 || rest < 0 || upper <= m_first || rest > NUM_CU / 2 + 8) return 0;
   return (int)m_first;
 }
 
@@ -1494,19 +1581,82 @@ static int launch_main_class(const S2SArgs& a, bool b_tr, hipStream_t st) {
 // loads, 1024 rows on average (a fifth of the tile rows partly filled, several experts below 128 rows) 5.76 -> 5.51 ms;
 // 128 experts of 2048 +- 45 rows 8.01 -> 7.97 ms; 8 experts of 4096 rows 29.36 -> 29.58 ms (the second launch costs
 // what it saves): taken below 1536 rows per expert.
+// With many rows per expert and few tile columns that second launch has too few workgroups for the chip and every one
+// of them walks the whole contraction (8 experts x 16 tile columns: 64 to 128 workgroups, as long as a full tile).
+// Plain products with a caller workspace then cut the contraction of those tiles into parts, one workgroup each
+// (tail_ksplit), and a small launch adds the parts up: float32 partial sums in a fixed order, so the result is the
+// same on every run, but no longer the same bits as the unsplit product (its additions are grouped differently).
 static constexpr double REMAINDER_MIN_FLOP = 2e11;
 static constexpr int REMAINDER_MAX_AVG_ROWS = 1536;
+static constexpr int KSPLIT_MAX = 8;
+static constexpr int KSPLIT_MIN_SLICES = 16;      // 64-deep slices a part must keep
+static constexpr int64_t SPLITK_TILE_FLOATS = 128 * 256;
+
+// Parts to cut the contraction of the last tiles into: enough for one workgroup per CU when half of the experts
+// have such a tile; 1 = not split (also: no workspace, fused unit behind the product, ragged contraction).
+static int tail_ksplit_for(int64_t K, int64_t N, int E, int glu) {
+  if (glu != 0 || K % BK != 0) return 1;
+  const int64_t n_tiles = (N + 255) / 256;
+  const int64_t wgs = std::max<int64_t>(1, (int64_t)(E + 1) / 2 * n_tiles);
+  int ks = 1;
+  while (ks < KSPLIT_MAX && wgs * ks < NUM_CU && K % (BK * ks * 2) == 0 && K / (BK * ks * 2) >= KSPLIT_MIN_SLICES) ks *= 2;
+  return ks;
+}
+static int64_t splitk_floats(int64_t N, int E, int ks) { return (int64_t)E * ((N + 255) / 256) * ks * SPLITK_TILE_FLOATS; }
+static int tail_ksplit(const S2SArgs& a) {
+  if (a.L / a.E < REMAINDER_MAX_AVG_ROWS) return 1;      // enough last tiles to fill the chip as they are
+  const int ks = tail_ksplit_for(a.K, a.N, a.E, a.glu);
+  if (ks <= 1 || a.partial == nullptr || a.partial_floats < splitk_floats(a.N, a.E, ks)) return 1;
+  return ks;
+}
+
+int64_t s2s_workspace_floats(int64_t L, int64_t K, int64_t N, int E, int dtype) {
+  if ((dtype != SMOE_BF16 && dtype != SMOE_F16) || E <= 0 || L / E < REMAINDER_MAX_AVG_ROWS) return 0;
+  if (2.0 * (double)L * K * N < REMAINDER_MIN_FLOP) return 0;
+  const int ks = tail_ksplit_for(K, N, E, 0);
+  return ks > 1 ? splitk_floats(N, E, ks) : 0;
+}
+
+static bool cut_tails(const S2SArgs& a) {
+  const bool whole = a.m_begin == 0 && a.m_count == 0x7fffffff && a.tail_mode == 0;
+  if (!whole || 2.0 * (double)a.L * a.K * (a.glu == 1 ? 2.0 * a.N : (double)a.N) < REMAINDER_MIN_FLOP) return false;
+  return a.L / a.E < REMAINDER_MAX_AVG_ROWS || tail_ksplit(a) > 1;
+}
+
+template <typename T>
+static int launch_tails(const S2SArgs& a, bool b_tr, hipStream_t st) {
+  typedef Tile<128, 256, 2, 4, 3> TailTile;
+  S2SArgs rest = a;
+  rest.tail_mode = 2;
+  rest.ksplit = tail_ksplit(a);
+  rest.k_part = a.K / rest.ksplit;
+  if (const int rc = launch_s2s<T, TailTile>(rest, b_tr, st)) return rc;
+  if (rest.ksplit <= 1) return 0;
+  const int n_tiles = (a.N + 255) / 256;
+  hipLaunchKernelGGL(splitk_reduce_kernel<T>, dim3((unsigned)n_tiles, (unsigned)a.E), dim3(512), 0, st, rest, n_tiles);
+  return launch_status("splitk_reduce_kernel");
+}
+
+// A whole product in the 256-row classes: the experts' sparsely filled last tiles apart (cut_tails), the rest as
+// whole rounds of 256 x 256 tiles plus a remainder of 256 x 128 tiles (tail_split) or as one launch.
 template <typename T>
 static int launch_main(const S2SArgs& a, bool b_tr, hipStream_t st) {
-  const bool whole = a.m_begin == 0 && a.m_count == 0x7fffffff && a.tail_mode == 0;
-  if (!whole || a.L / a.E >= REMAINDER_MAX_AVG_ROWS ||
-      2.0 * (double)a.L * a.K * (a.glu == 1 ? 2.0 * a.N : (double)a.N) < REMAINDER_MIN_FLOP)
-    return launch_main_class<T>(a, b_tr, st);
-  S2SArgs main = a, rest = a;
-  main.tail_mode = 1;
-  rest.tail_mode = 2;
-  if (const int rc = launch_main_class<T>(main, b_tr, st)) return rc;
-  return launch_s2s<T, Tile<128, 256, 2, 4, 3>>(rest, b_tr, st);
+  S2SArgs m = a;
+  const bool tails = cut_tails(a);
+  if (tails) m.tail_mode = 1;
+  int rc;
+  if (const int m_first = a.L / a.E >= ROWS256_BELOW ? tail_split(m) : 0) {
+    S2SArgs first = m, rest = m;
+    first.m_count = m_first;
+    rest.m_begin = m_first;
+    // both classes have 256-row tiles, hence the same numbering of the tile rows
+    rc = launch_main_class<T>(first, b_tr, st);
+    if (rc == 0) rc = launch_s2s<T, Tile<256, 128, 4, 2, 3>>(rest, b_tr, st);
+  } else {
+    rc = launch_main_class<T>(m, b_tr, st);
+  }
+  if (rc != 0 || !tails) return rc;
+  return launch_tails<T>(a, b_tr, st);
 }
 
 template <typename T>
@@ -1520,15 +1670,11 @@ static int dispatch_s2s(const S2SArgs& a, bool b_tr, hipStream_t st) {
   // the backward gated epilogues address a tile's output rows with 32-bit byte offsets from its first row
   if ((a.glu == 2 || a.glu == 4) && a.sym * 2 * 256 >= 0xffffffffLL) return SMOE_ERR_UNSUPPORTED;
   const int64_t avg = a.L / a.E;
-  if (const int m_first = avg >= ROWS256_BELOW ? tail_split(a) : 0) {
-    S2SArgs first = a, rest = a;
-    first.m_count = m_first;
-    rest.m_begin = m_first;
-    // both classes have 256-row tiles, hence the same numbering of the tile rows
-    if (const int rc = launch_main<T>(first, b_tr, st)) return rc;
-    return launch_s2s<T, Tile<256, 128, 4, 2, 3>>(rest, b_tr, st);
+  if (avg >= ROWS256_BELOW) {
+    S2SArgs m = a;
+    if (cut_tails(a)) m.tail_mode = 1;
+    if (tail_split(m) != 0 || !half_width_wins(a)) return launch_main<T>(a, b_tr, st);
   }
-  if (avg >= ROWS256_BELOW && !half_width_wins(a)) return launch_main<T>(a, b_tr, st);
   // Wide launches (enough 256-wide tile columns to fill the chip twice even with one tile row per expert, e.g.
   // Mixtral layer 1) move half as many token rows per weight byte with 256-wide tiles as with 128-wide ones:
   // the 256 x 256 class from 136 rows per expert on (544..832 Mixtral tokens: layer 1 -9..-11 % against the
@@ -1729,7 +1875,7 @@ static int launch_xty(const XtYArgs& a, hipStream_t st) {
 }
 
 bool try_xty_mfma(const XtYArgs& a, int dtype, hipStream_t st, int& rc) {
-  if (dtype == SMOE_F32) return try_xty_f32(a, st, rc);
+  if (dtype == SMOE_F32) return a.idx == nullptr && try_xty_f32(a, st, rc);    // the float32 kernels do not gather
   if (dtype != SMOE_BF16 && dtype != SMOE_F16) return false;
   if (a.K % 8 != 0 || a.N % 8 != 0) return false;
   if (a.sdyn != 1 || a.sxk != 1 || a.sdym % 8 != 0 || a.sxm % 8 != 0) return false;

@@ -300,6 +300,10 @@ int launch_route(const void* ids, int idx_dtype, int64_t L, int E, int64_t* eid_
 
 int launch_route_static(const void* ids, int idx_dtype, int64_t L, int E, int64_t* eid_out, int64_t* idx_out,
                         int64_t* off_out, hipStream_t st) {
+  if (E > kRouteMaxE) {          // before the buffer check: too many experts is a range error, not a workspace one
+    set_error("smoe_route_static: E=%d exceeds the supported maximum %d", E, kRouteMaxE);
+    return SMOE_ERR_RANGE;
+  }
   const size_t need = route_workspace_bytes(L, E);
   if (need > (size_t)SMOE_ROUTE_STATIC_BYTES) {
     set_error("smoe_route_static: L=%lld rows over E=%d experts need %zu bytes of histograms, the built-in buffer "

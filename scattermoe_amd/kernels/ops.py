@@ -51,16 +51,21 @@ class HipBackend:
         _C.require_gpu(X, "scatter2scatter")
         lib = _C.load()
         sbe, sbn = (b.stride(0), b.stride(1)) if b is not None else (0, 0)
+        code = _C.float_code(X.dtype)
+        # scratch for the products that split the contraction of their experts' last tiles (0 bytes for the others);
+        # torch's allocator hands the same block out again step after step
+        need = lib.smoe_scatter2scatter_workspace_bytes(eid.numel(), X.size(1), Y.size(1), W.size(0), code)
+        ws = torch.empty(need, dtype=torch.uint8, device=X.device) if need else None
         with _C.on_device(X.device):
-            rc = lib.smoe_scatter2scatter(
+            rc = lib.smoe_scatter2scatter_ws(
                 _C.ptr(X), X.stride(0), X.stride(1),
                 _C.ptr(W), W.stride(0), W.stride(1), W.stride(2),
                 _C.ptr(b), sbe, sbn,
                 _C.ptr(Y), Y.stride(0), Y.stride(1),
                 _C.ptr(eid), _C.ptr(idx), _C.ptr(off),
                 eid.numel(), X.size(1), Y.size(1), W.size(0), k,
-                int(bool(x_grouped)), int(bool(y_grouped)), _C.float_code(X.dtype),
-                _C.stream_ptr(X.device))
+                int(bool(x_grouped)), int(bool(y_grouped)), code,
+                _C.ptr(ws), need, _C.stream_ptr(X.device))
         _C.check(rc, "smoe_scatter2scatter")
 
     @staticmethod

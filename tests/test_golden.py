@@ -1,4 +1,5 @@
 """The committed c1 fixture: the oracle reproduces it on CPU, the HIP path reproduces it on the GPU."""
+import hashlib
 import json
 import os
 
@@ -9,6 +10,17 @@ import oracle
 from _inputs import CONFIGS, make_inputs
 
 FIX = json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "c1_seed0.json")))
+
+
+def _digest(t):
+    return hashlib.sha256(t.detach().contiguous().numpy().tobytes()).hexdigest()[:16]
+
+
+def test_inputs_are_the_ones_the_fixture_was_made_from():
+    """The expected rows mean something only for the inputs they were computed from: the seeded draw must still give
+    the tensors whose digests the fixture records."""
+    t = make_inputs(CONFIGS["c1"], seed=0)
+    assert {k: _digest(v) for k, v in t.items()} == FIX["inputs_sha256_16"]
 
 
 def _check(y, dx, dp, dw1, dw2, routing, tol):

@@ -203,6 +203,72 @@ def test_s2s_last_tiles_of_few_rows_in_their_own_launch(x_grouped, y_grouped):
     assert torch.equal(got, torch.cat(halves, 1))
 
 
+SPLIT_COUNTS = [1613, 1830, 1792, 2432, 60]      # last tiles of 77, 38, none, 128 rows; an expert of 60 rows only
+
+
+def _s2s_through_the_c_abi(X, W, b, eid, idx, off, fan, x_grouped, y_grouped, workspace):
+    """smoe_scatter2scatter_ws with the workspace the library asks for, or smoe_scatter2scatter (none)."""
+    from scattermoe_amd import _C
+    lib = _C.load()
+    L, N = eid.numel(), W.size(2)
+    Y = torch.full((L, N), float("nan"), dtype=X.dtype, device=DEV)
+    common = (_C.ptr(X), X.stride(0), X.stride(1), _C.ptr(W), W.stride(0), W.stride(1), W.stride(2),
+              _C.ptr(b), b.stride(0), b.stride(1), _C.ptr(Y), Y.stride(0), Y.stride(1), _C.ptr(eid), _C.ptr(idx),
+              _C.ptr(off), L, X.size(1), N, W.size(0), fan, int(x_grouped), int(y_grouped), _C.float_code(X.dtype))
+    if workspace:
+        need = lib.smoe_scatter2scatter_workspace_bytes(L, X.size(1), N, W.size(0), _C.float_code(X.dtype))
+        assert need > 0, "this product is meant to split the contraction of its last tiles"
+        ws = torch.empty(need, dtype=torch.uint8, device=DEV)
+        rc = lib.smoe_scatter2scatter_ws(*common, _C.ptr(ws), need, _C.stream_ptr(X.device))
+    else:
+        rc = lib.smoe_scatter2scatter(*common, _C.stream_ptr(X.device))
+    assert rc == 0, lib.smoe_last_error()
+    torch.cuda.synchronize()
+    return Y
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("w_layout", ["k_contig", "n_contig"])
+@pytest.mark.parametrize("x_grouped,y_grouped", [(False, True), (True, False), (True, True)])
+def test_s2s_last_tiles_with_split_contraction(x_grouped, y_grouped, w_layout, dtype):
+    """Many rows per expert, few tile columns and a long contraction (the Mixtral layer-2 forward and layer-1 input
+    gradient in small): with a workspace the experts' last tiles of at most 128 rows are multiplied in contraction
+    parts and added up by a second launch.  Against the oracle at the usual bar; the same bits on a second run (the
+    parts are added in a fixed order); and against the product without workspace: the same bits in every row outside
+    those tiles, within float32 regrouping of the sum (one unit in the last place of the 16-bit result) inside."""
+    counts, k, K, N = SPLIT_COUNTS, 1, 4096, 4096
+    E, L = len(counts), sum(counts)
+    eid, idx, off, g = _routing_with_counts(counts, k, seed=21)
+    X = torch.randn(L, K, generator=g).to(dtype)
+    Wp = (torch.randn(E, N, K, generator=g) * 0.03).to(dtype)
+    b = torch.randn(E, N, generator=g).to(dtype)
+    Wd = Wp.to(DEV).permute(0, 2, 1)
+    if w_layout == "n_contig":
+        Wd = Wd.contiguous()
+    args = (X.to(DEV), Wd, b.to(DEV), eid.to(DEV), idx.to(DEV), off.to(DEV), 1, x_grouped, y_grouped)
+    got = _s2s_through_the_c_abi(*args, workspace=True)
+    want = oracle.scatter2scatter_ref(X.float(), Wp.permute(0, 2, 1).float(), eid, idx, 1, b.float(), x_grouped, y_grouped)
+    _close(got, want, scale=0.03 * K ** 0.5)
+    assert torch.equal(got, _s2s_through_the_c_abi(*args, workspace=True))
+    plain = _s2s_through_the_c_abi(*args, workspace=False)
+    in_tail = torch.zeros(L, dtype=torch.bool)
+    lo = 0
+    for c in counts:
+        if 0 < c % 256 <= 128:
+            in_tail[lo + c - c % 256:lo + c] = True
+        lo += c
+    rows = in_tail if y_grouped else torch.zeros(L, dtype=torch.bool).index_put_((idx,), in_tail)
+    assert int(rows.sum()) == 77 + 38 + 128 + 60
+    assert torch.equal(got[~rows.to(DEV)], plain[~rows.to(DEV)])
+    a, p = got[rows.to(DEV)].float(), plain[rows.to(DEV)].float()
+    ulp = 2.0 ** (-7 if dtype == torch.bfloat16 else -10)
+    assert bool(((a - p).abs() <= ulp * p.abs() + 1e-4).all())      # float32 regrouping of a sum of 4096 terms of size 1
+    # the module-level wrapper brings the workspace by itself
+    via_ops = ops.scatter2scatter(args[0], Wd, args[3], args[4], 1, b=args[2], x_grouped=x_grouped, y_grouped=y_grouped,
+                                  expert_offsets=args[5])
+    assert torch.equal(via_ops, got)
+
+
 @pytest.mark.parametrize("act", ["SILU", "GPT_OSS"])
 def test_fused_gated_products_with_last_tiles_in_their_own_launch(act):
     """The same row counts through the products that carry the gated unit in their epilogue (forward: saved
@@ -237,7 +303,8 @@ def test_fused_gated_products_with_last_tiles_in_their_own_launch(act):
 
 
 @pytest.mark.parametrize("T,E,k,K,N", [(4000, 8, 2, 64, 4096),        # cut by tile rows: whole rounds + remainder
-                                       (5000, 8, 2, 2048, 7680)])     # experts' last tiles of few rows on their own
+                                       (5000, 8, 2, 2048, 7680),      # experts' last tiles of few rows on their own
+                                       (4100, 4, 2, 4096, 4096)])     # ... multiplied in contraction parts (workspace)
 def test_split_product_replays_from_a_graph(T, E, k, K, N):
     """A product that runs as two launches (see the tests above), routing included, captured into a HIP graph and
     replayed on fresh inputs (the routing, hence which tiles go to which launch, changes from replay to replay), with
