@@ -218,6 +218,25 @@ int smoe_gate_grad(const void* Y, int64_t sym, const void* dOut, int64_t sdm, vo
                    int64_t T, int k, int64_t N, int dtype, void* stream);
 
 /*
+ * smoe_gate_grad and the scaled gather of the output gradient in ONE pass over the expert outputs: the two steps with
+ * which the backward of a gate-weighted expert layer begins (scattermoe/parallel_experts.py:76-93:
+ * `d_gates = output_expanded @ grad_out` as a bmm, then `group(grad_out, sorted_scattered_idxs, fan_out=k,
+ * coeff=gates.flatten(), out=output_expanded)`).
+ *   dgates[t, j] = <Y[t*k + j, :], dOut[t, :]>            dY[inv[t*k + j], :] = dOut[t, :] * gates[t, j]
+ * with inv the inverse of the permutation idx (built by a first small launch in `inverse_workspace`, L = T*k int32).
+ * dOut is read from memory once instead of twice.  Unlike the reference's in-place reuse, dY must NOT overlap Y
+ * (row s of Y may still be unread when another row of dY is written).  Y (L,N) rows in slot order, dOut (T,N),
+ * gates (T,k) strides sgt,sgk, dY (L,N) in expert-sorted order, dgates (T,k) strides sdgt,sdgk; columns contiguous.
+ * A row whose index entry is shared or out of range is left unwritten (use smoe_gate_grad + smoe_group then).
+ * Returns SMOE_ERR_UNSUPPORTED (nothing launched) unless rows are whole 16-byte pieces and 16-byte aligned.
+ */
+int smoe_gate_grad_group(const void* Y, int64_t sym, const void* dOut, int64_t sdm,
+                         const void* gates, int64_t sgt, int64_t sgk,
+                         const int64_t* idx, int32_t* inverse_workspace,
+                         void* dY, int64_t sdym, void* dgates, int64_t sdgt, int64_t sdgk,
+                         int64_t T, int k, int64_t N, int dtype, void* stream);
+
+/*
  * Gated linear unit of GLUMLP in one pass:  h = act(pre[:, f:2f]) * pre[:, 0:f]   (first half linear,
  * second half activated), replacing chunk + activation + multiply of scattermoe/mlp.py:81-87, and its
  * gradient  dpre[:, 0:f] = dh * act(g),  dpre[:, f:2f] = dh * lin * act'(g)  that autograd derives from it.

@@ -44,6 +44,8 @@ _SIGNATURES = {
                                       _p, _i64, _i64, _i64, _int, _int, _p]),
     "smoe_combine": (_int, [_p, _i64, _p, _i64, _i64, _p, _i64, _i64, _int, _i64, _int, _p]),
     "smoe_gate_grad": (_int, [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _int, _i64, _int, _p]),
+    "smoe_gate_grad_group": (_int, [_p, _i64, _p, _i64, _p, _i64, _i64, _p, _p, _p, _i64, _p, _i64, _i64,
+                                    _i64, _int, _i64, _int, _p]),
     "smoe_glu_fwd": (_int, [_p, _i64, _p, _i64, _i64, _i64, _int, _int, _p]),
     "smoe_glu_bwd": (_int, [_p, _i64, _p, _i64, _p, _i64, _i64, _i64, _int, _int, _p]),
     "smoe_scatter2scatter_glu": (_int, [_p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _i64, _p, _i64, _p, _i64,

@@ -285,6 +285,20 @@ int smoe_gate_grad(const void* Y, int64_t sym, const void* dOut, int64_t sdm, vo
   return launch_gate_grad(Y, sym, dOut, sdm, dgates, sgt, sgk, T, k, (int)N, dtype, (hipStream_t)stream);
 }
 
+int smoe_gate_grad_group(const void* Y, int64_t sym, const void* dOut, int64_t sdm, const void* gates, int64_t sgt,
+                         int64_t sgk, const int64_t* idx, int32_t* inverse_workspace, void* dY, int64_t sdym,
+                         void* dgates, int64_t sdgt, int64_t sdgk, int64_t T, int k, int64_t N, int dtype, void* stream) {
+  g_err[0] = 0;
+  if (!dtype_ok(dtype)) { set_error("smoe_gate_grad_group: unknown dtype %d", dtype); return SMOE_ERR_DTYPE; }
+  if (T < 0 || k <= 0 || N < 0) { set_error("smoe_gate_grad_group: bad sizes"); return SMOE_ERR_SHAPE; }
+  if (T > 0x7fffffffLL || N > 0x7fffffffLL || T * k > 0x7fffffffLL) { set_error("smoe_gate_grad_group: size beyond int32"); return SMOE_ERR_RANGE; }
+  if (T == 0) return 0;
+  if (!Y || !dOut || !gates || !idx || !inverse_workspace || !dY || !dgates) { set_error("smoe_gate_grad_group: NULL pointer"); return SMOE_ERR_NULL; }
+  if (N == 0) return SMOE_ERR_UNSUPPORTED;
+  return launch_gate_grad_group(Y, sym, dOut, sdm, gates, sgt, sgk, idx, (int*)inverse_workspace, dY, sdym, dgates, sdgt,
+                                sdgk, T, k, (int)N, dtype, (hipStream_t)stream);
+}
+
 int smoe_glu_fwd(const void* pre, int64_t spm, void* h, int64_t shm, int64_t rows, int64_t f, int act, int dtype,
                  void* stream) {
   g_err[0] = 0;

@@ -273,6 +273,12 @@ int launch_route_static(const void* expert_idxs, int idx_dtype, int64_t L, int E
 int route_static_init();
 int launch_offsets_from_sorted(const int64_t* eid, int64_t L, int E, int64_t* off, hipStream_t st);
 int launch_group_by_source(const GroupArgs& a, int* inv, int dtype, hipStream_t st);
+int launch_invert_index(const int64_t* idx, int64_t L, int* inv, hipStream_t st);   // inv[idx[r]] = r
+// gate gradient and the scaled, expert-sorted copy of the output gradient in one pass (csrc/fused.hip);
+// SMOE_ERR_UNSUPPORTED when rows are not 16-byte pieces
+int launch_gate_grad_group(const void* Y, int64_t sy, const void* D, int64_t sd, const void* G, int64_t sgt, int64_t sgk,
+                           const int64_t* idx, int* inv, void* DY, int64_t sdy, void* DG, int64_t sdgt, int64_t sdgk,
+                           int64_t Tn, int k, int N, int dtype, hipStream_t st);
 int launch_mfma_rate_probe(float* out, int iters, int random_operands, double* flop, hipStream_t st);
 
 }  // namespace smoe

@@ -116,6 +116,65 @@ __global__ __launch_bounds__(256) void gate_grad_kernel(const T* __restrict__ Y,
   }
 }
 
+// ---- gate gradient + scaled gather of the output gradient, one pass ------------------------------------
+// The backward pass of a gate-weighted expert layer walks the (L, N) expert outputs for the gate gradient and
+// writes an (L, N) matrix of scaled output-gradient rows in expert-sorted order (reference parallel_experts.py:
+// 76-93: a bmm, then group with coefficients).  Here one wave owns one (token, slot) row s = t * k + j: it reads
+// dOut[t] (its k readers run side by side, so the memory side sees it once) and Y[s], adds up their dot product,
+// and writes dOut[t] * gates[t, j] to row inv[s] of dY - which therefore is a buffer of its own: row s of Y may
+// still be unread when some other wave's row of dY lands on it.  inv = inverse of the routing permutation
+// (launch_invert_index); a row whose inverse entry does not point back at it is not written, as in
+// group_by_source.  The product dOut * gate is rounded once, like group's; the dot product is added up in float32
+// by one wave in a fixed order.
+template <typename T, int P>
+__global__ __launch_bounds__(256) void gate_grad_group_kernel(const T* __restrict__ Y, int64_t sy, const T* __restrict__ D,
+                                                             int64_t sd, const T* __restrict__ G, int64_t sgt, int64_t sgk,
+                                                             const int64_t* __restrict__ idx, const int* __restrict__ inv,
+                                                             T* __restrict__ DY, int64_t sdy, T* __restrict__ DG,
+                                                             int64_t sdgt, int64_t sdgk, int64_t L, int k, int N) {
+  typedef Pack<T> V;
+  const int lane = lane_id(), wave = threadIdx.x >> 6;
+  const int nv = N / V::n;
+  for (int64_t s = (int64_t)blockIdx.x * 4 + wave; s < L; s += (int64_t)gridDim.x * 4) {
+    const int64_t t = s / k;
+    const int j = (int)(s - t * k);
+    const int q = inv[s];
+    const bool mine = (unsigned)q < (uint64_t)L && idx[q] == s;
+    const float c = to_f32(G[t * sgt + j * sgk]);
+    const T* __restrict__ y = Y + s * sy;
+    const T* __restrict__ d = D + t * sd;
+    T* __restrict__ o = DY + (int64_t)(mine ? q : 0) * sdy;
+    float acc = 0.0f;
+    for (int j0 = 0; j0 < nv; j0 += 64 * P) {
+      V a[P], b[P];
+#pragma unroll
+      for (int p = 0; p < P; ++p) {
+        const int c16 = j0 + p * 64 + lane;
+        if (c16 < nv) {
+          a[p] = stream_load16<V>(y + (int64_t)c16 * V::n);
+          b[p] = *(const V*)(d + (int64_t)c16 * V::n);
+        }
+      }
+#pragma unroll
+      for (int p = 0; p < P; ++p) {
+        const int c16 = j0 + p * 64 + lane;
+        if (c16 >= nv) continue;
+        V w;
+#pragma unroll
+        for (int e = 0; e < V::n; ++e) {
+          const float dv = to_f32(b[p].v[e]);
+          acc = fmaf(to_f32(a[p].v[e]), dv, acc);
+          w.v[e] = from_f32<T>(dv * c);
+        }
+        if (mine) stream_store16(o + (int64_t)c16 * V::n, w);
+      }
+    }
+#pragma unroll
+    for (int sh = 32; sh > 0; sh >>= 1) acc += __shfl_xor(acc, sh, 64);
+    if (lane == 0) DG[t * sdgt + j * sdgk] = from_f32<T>(acc);
+  }
+}
+
 // ---- gated linear unit -----------------------------------------------------------------------------------
 // sigmoidf_, act_f, act_df: common.hpp
 
@@ -276,6 +335,22 @@ static int glu_bwd_t(const void* pre, int64_t sp, const void* dh, int64_t sdh, v
   return launch_status("glu_bwd_kernel");
 }
 
+template <typename T>
+static int gate_grad_group_t(const void* Y, int64_t sy, const void* D, int64_t sd, const void* G, int64_t sgt, int64_t sgk,
+                             const int64_t* idx, int* inv, void* DY, int64_t sdy, void* DG, int64_t sdgt, int64_t sdgk,
+                             int64_t Tn, int k, int N, hipStream_t st) {
+  constexpr int vn = 16 / sizeof(T);
+  const bool vec = N % vn == 0 && sy % vn == 0 && sd % vn == 0 && sdy % vn == 0 && al16(Y) && al16(D) && al16(DY);
+  const int64_t L = Tn * k;
+  if (!vec || L > 0x7fffffffLL) return SMOE_ERR_UNSUPPORTED;
+  if (const int rc = launch_invert_index(idx, L, inv, st)) return rc;
+  int64_t blocks = cdiv64(L, 4);
+  if (blocks > 256 * 64) blocks = 256 * 64;
+  hipLaunchKernelGGL((gate_grad_group_kernel<T, 4>), dim3((unsigned)blocks), dim3(256), 0, st, (const T*)Y, sy, (const T*)D, sd,
+                     (const T*)G, sgt, sgk, idx, (const int*)inv, (T*)DY, sdy, (T*)DG, sdgt, sdgk, L, k, N);
+  return launch_status("gate_grad_group_kernel");
+}
+
 #define SMOE_DISPATCH(dtype, CALL)                                              \
   switch (dtype) {                                                              \
     case SMOE_F32: { typedef float T; return CALL; }                            \
@@ -291,6 +366,11 @@ int launch_combine(const void* Y, int64_t sy, const void* G, int64_t sgt, int64_
 int launch_gate_grad(const void* Y, int64_t sy, const void* D, int64_t sd, void* DG, int64_t sgt, int64_t sgk,
                      int64_t Tn, int k, int N, int dtype, hipStream_t st) {
   SMOE_DISPATCH(dtype, gate_grad_t<T>(Y, sy, D, sd, DG, sgt, sgk, Tn, k, N, st));
+}
+int launch_gate_grad_group(const void* Y, int64_t sy, const void* D, int64_t sd, const void* G, int64_t sgt, int64_t sgk,
+                           const int64_t* idx, int* inv, void* DY, int64_t sdy, void* DG, int64_t sdgt, int64_t sdgk,
+                           int64_t Tn, int k, int N, int dtype, hipStream_t st) {
+  SMOE_DISPATCH(dtype, gate_grad_group_t<T>(Y, sy, D, sd, G, sgt, sgk, idx, inv, DY, sdy, DG, sdgt, sdgk, Tn, k, N, st));
 }
 int launch_glu_fwd(const void* pre, int64_t sp, void* h, int64_t sh, int64_t rows, int f, int act, int dtype, hipStream_t st) {
   SMOE_DISPATCH(dtype, glu_fwd_t<T>(pre, sp, h, sh, rows, f, act, st));

@@ -76,6 +76,12 @@ __global__ __launch_bounds__(256) void invert_index_kernel(const int64_t* __rest
   if ((uint64_t)s < (uint64_t)L) inv[s] = r;
 }
 
+int launch_invert_index(const int64_t* idx, int64_t L, int* inv, hipStream_t st) {
+  if (L == 0) return 0;
+  hipLaunchKernelGGL(invert_index_kernel, dim3((unsigned)cdiv64(L, 256)), dim3(256), 0, st, idx, (int)L, inv);
+  return launch_status("invert_index_kernel");
+}
+
 template <typename T, int P>
 __global__ __launch_bounds__(kGroupThreads) void group_by_source_kernel(GroupArgs a, const int* __restrict__ inv) {
   typedef Vec16<T> V;

@@ -151,6 +151,21 @@ class HipBackend:
         _C.check(rc, "smoe_gate_grad")
 
     @staticmethod
+    def gate_grad_group(Y, d_out, gates, idx, inverse, dy, d_gates, k):
+        """Gate gradient + scaled expert-sorted copy of d_out in one pass; False if the library declines."""
+        _C.require_gpu(Y, "gate_grad_group")
+        lib = _C.load()
+        with _C.on_device(Y.device):
+            rc = lib.smoe_gate_grad_group(_C.ptr(Y), Y.stride(0), _C.ptr(d_out), d_out.stride(0),
+                                          _C.ptr(gates), gates.stride(0), gates.stride(1), _C.ptr(idx), _C.ptr(inverse),
+                                          _C.ptr(dy), dy.stride(0), _C.ptr(d_gates), d_gates.stride(0), d_gates.stride(1),
+                                          d_out.size(0), k, Y.size(1), _C.float_code(Y.dtype), _C.stream_ptr(Y.device))
+        if rc == _C.ERR_UNSUPPORTED:
+            return False
+        _C.check(rc, "smoe_gate_grad_group")
+        return True
+
+    @staticmethod
     def glu_fwd(pre, h, act):
         _C.require_gpu(pre, "glu_fwd")
         lib = _C.load()
@@ -320,6 +335,20 @@ def _combine_op(Y: torch.Tensor, gates: Optional[torch.Tensor], out: torch.Tenso
 @torch.library.custom_op("scattermoe::gate_grad", mutates_args={"d_gates"})
 def _gate_grad_op(Y: torch.Tensor, d_out: torch.Tensor, d_gates: torch.Tensor, k: int) -> None:
     _backend.gate_grad(Y, d_out, d_gates, k)
+
+
+@torch.library.custom_op("scattermoe::gate_grad_group", mutates_args={"dy", "d_gates"})
+def _gate_grad_group_op(Y: torch.Tensor, d_out: torch.Tensor, gates: torch.Tensor, idx: torch.Tensor, dy: torch.Tensor,
+                        d_gates: torch.Tensor, k: int) -> None:
+    _gate_grad_group_launch(Y, d_out, gates, idx, dy, d_gates, k)
+
+
+def _gate_grad_group_launch(Y, d_out, gates, idx, dy, d_gates, k):
+    inverse = torch.empty(idx.numel(), dtype=torch.int32, device=Y.device)
+    if not (hasattr(_backend, "gate_grad_group")
+            and _backend.gate_grad_group(Y, d_out, gates, idx, inverse, dy, d_gates, k)):
+        _backend.gate_grad(Y, d_out, d_gates, k)                       # the two passes it stands for
+        _group_launch(d_out, dy, gates.reshape(-1), k, idx, True)
 
 
 @torch.library.custom_op("scattermoe::glu_fwd", mutates_args={"h"})
@@ -602,6 +631,28 @@ def gate_grad(expanded, grad_out):
     d_gates = torch.empty((T, k), dtype=expanded.dtype, device=expanded.device)
     _launch("gate_grad", Y, _rows_contiguous(grad_out), d_gates, k)
     return d_gates
+
+
+def gate_grad_group(expanded, grad_out, gates, sorted_scattered_idxs):
+    """(d_gates, dy): `gate_grad(expanded, grad_out)` and `group(grad_out, idxs, coeff=gates.flatten(), fan_out=k)`
+    - the first two steps of the backward of a gate-weighted expert layer (reference parallel_experts.py:76-93) -
+    in one pass that reads grad_out from memory once.  dy is a new (T * k, N) buffer in expert-sorted order (the
+    reference reuses the buffer of `expanded`, which a single pass cannot: it reads and writes different rows at the
+    same time).  `sorted_scattered_idxs` must be the routing's permutation of range(T * k)."""
+    T, k, N = expanded.shape
+    assert grad_out.shape == (T, N) and gates.shape == (T, k) and sorted_scattered_idxs.numel() == T * k
+    Y = _rows_contiguous(expanded.reshape(T * k, N))
+    d_out = _rows_contiguous(grad_out)
+    g = gates.to(expanded.dtype)
+    idx = _as_i64(sorted_scattered_idxs).contiguous()
+    dy = torch.empty((T * k, N), dtype=expanded.dtype, device=expanded.device)
+    d_gates = torch.empty((T, k), dtype=expanded.dtype, device=expanded.device)
+    if torch.compiler.is_compiling():
+        _gate_grad_group_op(Y, d_out, g, idx, dy, d_gates, k)
+    else:
+        _same_dtype("gate_grad_group", Y, d_out)
+        _gate_grad_group_launch(Y, d_out, g, idx, dy, d_gates, k)
+    return d_gates, dy
 
 
 def glu_fwd(pre, act=ACT_SILU):

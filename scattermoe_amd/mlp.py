@@ -59,10 +59,15 @@ class _GatedMLP(torch.autograd.Function):
         E = w1.size(0)
         if not grad_out.is_contiguous():
             grad_out = grad_out.contiguous()
-        d_gates = ops.gate_grad(kept, grad_out) if need_g else None
-        # dY of layer 2 in expert-sorted order, scaled by each row's gate; reuses the expert-output buffer
-        dy = ops.group(grad_out, idx, coeff=gates.reshape(-1).to(grad_out.dtype), fan_out=k, permutation=True,
-                       out=kept.view(-1, kept.size(-1)))
+        if need_g:
+            # gate gradient and dY of layer 2 (expert-sorted, scaled by each row's gate) in one pass over the
+            # expert outputs
+            d_gates, dy = ops.gate_grad_group(kept, grad_out, gates, idx)
+        else:
+            # dY alone reuses the expert-output buffer
+            d_gates = None
+            dy = ops.group(grad_out, idx, coeff=gates.reshape(-1).to(grad_out.dtype), fan_out=k, permutation=True,
+                           out=kept.view(-1, kept.size(-1)))
         d_w2 = d_b2 = None
         if need_w2 or need_b2:
             d_w2, d_b2 = ops.group_bwd_W(DY=dy, X=h, expert_offsets=off, E=E, has_bias=b2 is not None, like=w2)

@@ -77,11 +77,14 @@ class ParallelLinear(torch.autograd.Function):
         if not grad_out.is_contiguous():
             grad_out = grad_out.contiguous()
 
-        d_gates = None
+        d_gates = dy = None
         coeff, coeff_fan, dy_buf = None, 1, None
         if gates is not None:
-            if need_g:
-                # (T, k): row dots of every expert output with dY
+            if need_g and not grouped_out:
+                # (T, k) row dots of every expert output with dY, and dY in expert-sorted order scaled by the gate
+                # of each (token, slot), in one pass
+                d_gates, dy = ops.gate_grad_group(kept, grad_out, gates, idx)
+            elif need_g:
                 d_gates = ops.gate_grad(kept, grad_out)
             coeff, coeff_fan = gates.reshape(-1), gates.size(1)
             dy_buf = kept.view(-1, kept.size(-1))   # its contents are dead once d_gates exists
@@ -89,7 +92,7 @@ class ParallelLinear(torch.autograd.Function):
         # dY in expert-sorted order, scaled by the gate of each (token, slot)
         if grouped_out:
             dy = grad_out
-        else:
+        elif dy is None:
             dy = ops.group(grad_out, idx, coeff=coeff, fan_out=coeff_fan, out=dy_buf, permutation=True)
 
         d_w = d_b = None

@@ -248,6 +248,29 @@ def test_combine_and_gate_grad(T, k, N, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,k,N,E", [(1, 2, 128, 4), (300, 3, 104, 8), (1024, 2, 4096, 8), (77, 8, 264, 32),
+                                     (50, 1, 64, 4), (513, 4, 2880, 32), (40, 2, 100, 4)])
+def test_gate_grad_and_scaled_gather_in_one_pass(T, k, N, E, dtype):
+    """`gate_grad_group` = `gate_grad` + `group(grad_out, idx, coeff=gates, fan_out=k)` over one read of grad_out:
+    the gathered rows bit-exact against the oracle's group (one rounding of the product), the gate gradient against
+    the float32 row dots; rows longer than one pass of a wave (4096, 2880), rows that are no whole 16-byte pieces
+    (N = 100 with 16-bit types: the two separate passes run instead)."""
+    g = torch.Generator().manual_seed(T + N + k)
+    experts = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)])
+    _, idx, _ = oracle.route_ref(experts, E)
+    Y = torch.randn(T, k, N, generator=g).to(dtype)
+    gates = torch.rand(T, k, generator=g).to(dtype)
+    dO = torch.randn(T, N, generator=g).to(dtype)
+    d_gates, dy = ops.gate_grad_group(Y.to(DEV), dO.to(DEV), gates.to(DEV), idx.to(DEV))
+    want_dy = oracle.group_ref(dO, idx, gates.reshape(-1), k)
+    assert torch.equal(dy.cpu(), want_dy)
+    want_g = (Y.float() * dO.float().unsqueeze(1)).sum(-1)
+    _close(d_gates, want_g, dtype, scale=N ** 0.5)
+    again = ops.gate_grad_group(Y.to(DEV), dO.to(DEV), gates.to(DEV), idx.to(DEV))
+    assert torch.equal(again[0], d_gates) and torch.equal(again[1], dy)           # fixed summation order
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("rows,f", [(1, 128), (333, 100), (4096, 768), (64, 2880)])
 def test_glu_fwd_bwd(rows, f, dtype):
     g = torch.Generator().manual_seed(rows + f)

@@ -141,14 +141,26 @@ def test_product_path_refuses_cpu_tensors():
 
 @pytest.mark.parametrize("glu", [False, True])
 def test_second_backward_over_a_consumed_graph_is_refused(cpu_backend, glu):
-    """Backward reuses the saved expert-output buffer for the grouped output gradient.  A second backward over
-    the same graph must not silently read the overwritten buffer: like the reference, whose `group` op declares
-    the buffer as mutated (scattermoe/kernels/ops.py:389), it has to raise."""
+    """Without gate gradients, backward reuses the saved expert-output buffer for the grouped output gradient.  A
+    second backward over the same graph must not silently read the overwritten buffer: like the reference, whose
+    `group` op declares the buffer as mutated (scattermoe/kernels/ops.py:389), it has to raise."""
     m, x, p, experts, dy = _case(16, 32, 24, 4, 2, False, glu)
-    y = m(x, p, experts)
+    y = m(x, p.detach(), experts)
     y.backward(dy, retain_graph=True)
     with pytest.raises(RuntimeError, match="modified by an inplace operation"):
         y.backward(dy)
+
+
+@pytest.mark.parametrize("glu", [False, True])
+def test_second_backward_with_gate_gradients_repeats_the_first(cpu_backend, glu):
+    """With gate gradients the grouped output gradient gets a buffer of its own (it is written in the pass that
+    still reads the expert outputs), so the saved tensors stay intact and a retained graph can be walked again."""
+    m, x, p, experts, dy = _case(16, 32, 24, 4, 2, False, glu)
+    y = m(x, p, experts)
+    first = torch.autograd.grad(y, [x, p, m.experts.weight], dy, retain_graph=True)
+    second = torch.autograd.grad(y, [x, p, m.experts.weight], dy)
+    for a, b in zip(first, second):
+        assert torch.equal(a, b)
 
 
 def test_slot_sum_is_the_gateless_combine(cpu_backend):
