@@ -11,6 +11,13 @@ What each function follows in the reference (shawntan/scattermoe):
   naive_expert_forward the same sum regrouped per expert (gather rows -> 2 linears -> weighted index_add)
   glu / gpt_oss_glu    scattermoe/mlp.py:81-87 ; scattermoe/utils/replace_moe.py:39-43
   topk_softmax_ref     scattermoe/utils/replace_moe.py:67-71  softmax in float -> topk -> renormalise
+  rounded_glu_token_step, rounded_glu_hidden_unit_grads
+                       the forward + backward dataflow of scattermoe/mlp.py:74-95 and
+                       scattermoe/parallel_experts.py:36-134 written out by hand (no autograd), with every tensor the
+                       reference materialises in the storage type (layer-1 output, hidden, expanded layer-2 output,
+                       gate-scaled grad_out, d hidden, d layer-1 output, expanded d input, and every result) rounded
+                       to that type and float32 accumulation in between: what a bf16 run of the reference computes,
+                       up to summation order
 
 How it is pinned (tests/test_oracle.py): the reference stores no golden vectors (its single test
 compares two live computations on unseeded inputs, tests/test_mlp.py:46-49), so every function is
@@ -29,6 +36,7 @@ __all__ = [
     "route_ref", "scatter2scatter_ref", "group_ref", "group_bwd_W_ref",
     "naive_token_forward", "naive_expert_forward", "glu", "gpt_oss_glu",
     "module_params", "naive_module_forward", "topk_softmax_ref",
+    "rounded_glu_token_step", "rounded_glu_hidden_unit_grads",
 ]
 
 
@@ -164,3 +172,87 @@ def naive_module_forward(m, x, p, experts, per_token=False):
     hidden = glu(m.activation) if W1.size(1) == 2 * W2.size(2) and type(m).__name__ == "GLUMLP" else m.activation
     f = naive_token_forward if per_token else naive_expert_forward
     return f(x, p, experts, W1, W2, hidden, b1, b2)
+
+
+# ---------------------------------------------------------------------------------------------------
+# The GLU MoE MLP step with the storage type's rounding where the reference materialises a tensor.
+# Written out by hand, forward and backward; with dtype=torch.float32 nothing is rounded and the results
+# are the autograd gradients of naive_token_forward / naive_expert_forward (tests/test_oracle.py pins that).
+# Inputs are float32 tensors holding values of the storage type.
+# ---------------------------------------------------------------------------------------------------
+def _silu_parts(gat):
+    s = torch.sigmoid(gat)
+    return gat * s, s * (1.0 + gat * (1.0 - s))          # silu(g), silu'(g)
+
+
+def rounded_glu_token_step(x, p, experts, W1, W2, dy, dtype, b1=None, b2=None):
+    """(y, dx, dp) of the given tokens.  x (n, d), p / experts (n, k), dy (n, d); W1 (E, 2f, d), W2 (E, d, f)."""
+    rnd = lambda t: t.to(dtype).float()
+    n, k = experts.shape
+    f = W2.size(2)
+    y, dx, dp = torch.zeros_like(x), torch.zeros_like(x), torch.zeros_like(p)
+    for t in range(n):
+        out = torch.zeros(x.size(1))
+        parts = []
+        for j in range(k):
+            e = int(experts[t, j])
+            pre = W1[e] @ x[t]
+            if b1 is not None:
+                pre = pre + b1[e]
+            pre = rnd(pre)                                           # layer-1 output as stored
+            lin, gat = pre[:f], pre[f:]
+            a, da = _silu_parts(gat)
+            h = rnd(a * lin)                                         # hidden as stored
+            yj = W2[e] @ h
+            if b2 is not None:
+                yj = yj + b2[e]
+            yj = rnd(yj)                                             # expanded layer-2 output as stored
+            out = out + p[t, j] * yj                                 # float32, slot order
+            parts.append((e, lin, a, da, yj))
+        y[t] = rnd(out)
+        acc = torch.zeros(x.size(1))
+        for j, (e, lin, a, da, yj) in enumerate(parts):
+            dp[t, j] = rnd(torch.dot(yj, dy[t]))
+            gdy = rnd(dy[t] * p[t, j])                               # gate-scaled output gradient as stored
+            dh = rnd(W2[e].T @ gdy)                                  # d hidden as stored
+            dpre = torch.cat([rnd(dh * a), rnd((dh * lin) * da)])    # d layer-1 output as stored
+            acc = acc + rnd(W1[e].T @ dpre)                          # expanded d input as stored, summed in float32
+        dx[t] = rnd(acc)
+    return y, dx, dp
+
+
+def rounded_glu_hidden_unit_grads(x, p, experts, W1s, W2s, dy, dtype, b1s=None, with_b2=False):
+    """(dW1s, dW2s, db1s, db2) for a model cut down to a subset S of hidden units: W1s (E, 2|S|, d) holds the rows
+    S and f + S of W1, W2s (E, d, |S|) the columns S of W2 (a hidden unit's weight gradients depend on the other
+    units only through dy, which is given).  All tokens, all experts."""
+    rnd = lambda t: t.to(dtype).float()
+    E, k = W1s.size(0), experts.size(1)
+    ns = W2s.size(2)
+    _, idx, off = route_ref(experts, E)
+    tok = idx // k
+    gdy = rnd(dy[tok] * p.reshape(-1)[idx].unsqueeze(-1))            # expert-sorted, gate-scaled, as stored
+    dW1s, dW2s = torch.zeros_like(W1s), torch.zeros_like(W2s)
+    db1s = torch.zeros(E, 2 * ns) if b1s is not None else None
+    db2 = torch.zeros(E, x.size(1)) if with_b2 else None
+    lo = 0
+    for e in range(E):
+        hi = int(off[e])
+        if hi > lo:
+            xe, ge = x[tok[lo:hi]], gdy[lo:hi]
+            pre = xe @ W1s[e].T
+            if b1s is not None:
+                pre = pre + b1s[e]
+            pre = rnd(pre)
+            lin, gat = pre[:, :ns], pre[:, ns:]
+            a, da = _silu_parts(gat)
+            h = rnd(a * lin)
+            dh = rnd(ge @ W2s[e])
+            dpre = torch.cat([rnd(dh * a), rnd((dh * lin) * da)], dim=1)
+            dW1s[e] = rnd(dpre.T @ xe)
+            dW2s[e] = rnd(ge.T @ h)
+            if db1s is not None:
+                db1s[e] = rnd(dpre.sum(0))
+            if db2 is not None:
+                db2[e] = rnd(ge.sum(0))
+        lo = hi
+    return dW1s, dW2s, db1s, db2

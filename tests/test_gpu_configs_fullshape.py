@@ -13,7 +13,10 @@ The oracle cannot run a whole c2 / c3 / c4 step in seconds, but two exact reduct
 Routing, tokens and dY come from `_inputs.make_inputs` (CPU generator, seed 0, the draw order of the benchmark
 definition); the weights of these shapes are drawn on the device (seed 1) because drawing up to 5.6e9 normal
 numbers on the host takes longer than everything else in this file together.
-Bars: `_tol.check` (bf16 rel 2e-2 / abs 1e-2, absolute term scaled by the reference magnitude when that exceeds 1).
+Bars: `_tol.check` (bf16 rel 2e-2 / abs 1e-2, absolute term scaled by the reference magnitude when that exceeds 1)
+against the float32 oracle, and the literal bar (nothing scaled) against the oracle that rounds to the storage type
+wherever the path stores a tensor (`oracle.rounded_glu_token_step`, `oracle.rounded_glu_hidden_unit_grads`): the
+first bounds format error + kernel error, the second kernel error alone.
 """
 import pytest
 import torch
@@ -60,6 +63,12 @@ def _check_tokens(cfg, t, m, x, p, y, n_tokens, seed):
     check("%s Y (sampled tokens)" % cfg.name, y.detach()[toks.to(DEV)], want, cfg.dtype)
     check("%s dX (sampled tokens)" % cfg.name, x.grad[toks.to(DEV)], xs.grad, cfg.dtype)
     check("%s dgates (sampled tokens)" % cfg.name, p.grad[toks.to(DEV)], ps.grad, cfg.dtype)
+    # the same step with every tensor the path stores rounded to the storage type: what is left to differ is the
+    # order of the float32 sums, so the bar is the literal one (abs 1e-2, rel 2e-2, nothing scaled)
+    ry, rdx, rdp = oracle.rounded_glu_token_step(xs.detach(), ps.detach(), t["experts"][toks], W1, W2, dys, cfg.dtype, b1, b2)
+    check("%s Y vs rounded oracle" % cfg.name, y.detach()[toks.to(DEV)], ry, cfg.dtype, literal=True)
+    check("%s dX vs rounded oracle" % cfg.name, x.grad[toks.to(DEV)], rdx, cfg.dtype, literal=True)
+    check("%s dgates vs rounded oracle" % cfg.name, p.grad[toks.to(DEV)], rdp, cfg.dtype, literal=True)
 
 
 def _check_hidden_units(cfg, t, m, x, p, n_units, seed):
@@ -81,6 +90,14 @@ def _check_hidden_units(cfg, t, m, x, p, n_units, seed):
     if cfg.bias:
         check("%s db1 (sampled hidden units)" % cfg.name, m.experts.bias.grad[:, S2.to(DEV)], b1.grad, cfg.dtype)
         check("%s db2" % cfg.name, m.output_experts.bias.grad, b2.grad, cfg.dtype)
+    r1, r2, rb1, rb2 = oracle.rounded_glu_hidden_unit_grads(
+        xc, pc, t["experts"], W1.detach(), W2.detach(), t["dy"].to(cfg.dtype).float(), cfg.dtype,
+        b1.detach() if cfg.bias else None, with_b2=cfg.bias)
+    check("%s dW1 vs rounded oracle" % cfg.name, m.experts.weight.grad[:, S2.to(DEV)], r1, cfg.dtype, literal=True)
+    check("%s dW2 vs rounded oracle" % cfg.name, m.output_experts.weight.grad[:, :, S.to(DEV)], r2, cfg.dtype, literal=True)
+    if cfg.bias:
+        check("%s db1 vs rounded oracle" % cfg.name, m.experts.bias.grad[:, S2.to(DEV)], rb1, cfg.dtype, literal=True)
+        check("%s db2 vs rounded oracle" % cfg.name, m.output_experts.bias.grad, rb2, cfg.dtype, literal=True)
 
 
 def _check_routing(cfg, t):

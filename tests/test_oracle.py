@@ -292,3 +292,49 @@ def test_topk_softmax_hand_worked_and_ties():
     # k = E without renormalisation is the whole softmax, sorted
     w, i = oracle.topk_softmax_ref(logits, 4, renormalize=False)
     assert abs(float(w.sum()) - 1.0) < 1e-6 and i.tolist() == [[3, 2, 1, 0]]
+
+
+# ---------------------------------------------------------------------------------------------------
+# the hand-written forward + backward with storage-type rounding: without rounding (float32) it must be the autograd
+# gradient of the naive forms; with rounding it must stay within the format's error of them
+# ---------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("bias", [False, True])
+def test_rounded_step_without_rounding_is_autograd_of_the_naive_forms(bias):
+    g = torch.Generator().manual_seed(5)
+    T, d, f, E, k = 40, 24, 16, 4, 2
+    x, dy = torch.randn(T, d, generator=g), torch.randn(T, d, generator=g)
+    experts = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)])
+    p = torch.rand(T, k, generator=g)
+    W1, W2 = torch.randn(E, 2 * f, d, generator=g) * 0.3, torch.randn(E, d, f, generator=g) * 0.3
+    b1 = torch.randn(E, 2 * f, generator=g) * 0.3 if bias else None
+    b2 = torch.randn(E, d, generator=g) * 0.3 if bias else None
+    leaves = [t.clone().requires_grad_() for t in (x, p, W1, W2)] + ([b1.clone().requires_grad_(), b2.clone().requires_grad_()] if bias else [])
+    want_y = oracle.naive_expert_forward(leaves[0], leaves[1], experts, leaves[2], leaves[3], oracle.glu(torch.nn.SiLU()),
+                                         *(leaves[4:] if bias else []))
+    grads = torch.autograd.grad(want_y, leaves, dy)
+    y, dx, dp = oracle.rounded_glu_token_step(x, p, experts, W1, W2, dy, torch.float32, b1, b2)
+    assert torch.allclose(y, want_y.detach(), atol=1e-5)
+    assert torch.allclose(dx, grads[0], atol=1e-5) and torch.allclose(dp, grads[1], atol=1e-5)
+    S = torch.tensor([1, 5, 6, 15])
+    S2 = torch.cat([S, f + S])
+    dW1s, dW2s, db1s, db2 = oracle.rounded_glu_hidden_unit_grads(x, p, experts, W1[:, S2], W2[:, :, S], dy, torch.float32,
+                                                                b1[:, S2] if bias else None, with_b2=bias)
+    assert torch.allclose(dW1s, grads[2][:, S2], atol=1e-5) and torch.allclose(dW2s, grads[3][:, :, S], atol=1e-5)
+    if bias:
+        assert torch.allclose(db1s, grads[4][:, S2], atol=1e-5) and torch.allclose(db2, grads[5], atol=1e-5)
+
+
+def test_rounded_step_in_bfloat16_stays_within_the_format_error():
+    g = torch.Generator().manual_seed(6)
+    T, d, f, E, k = 32, 64, 48, 4, 2
+    bf = lambda t: t.bfloat16().float()
+    x, dy = bf(torch.randn(T, d, generator=g)), bf(torch.randn(T, d, generator=g))
+    experts = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)])
+    p = bf(torch.rand(T, k, generator=g))
+    W1, W2 = bf(torch.randn(E, 2 * f, d, generator=g) * 0.1), bf(torch.randn(E, d, f, generator=g) * 0.1)
+    exact = oracle.rounded_glu_token_step(x, p, experts, W1, W2, dy, torch.float32)
+    rounded = oracle.rounded_glu_token_step(x, p, experts, W1, W2, dy, torch.bfloat16)
+    for a, b in zip(exact, rounded):
+        assert torch.equal(b, bf(b))                                             # results are values of the format
+        assert float((a - b).abs().max()) <= 2e-2 * float(a.abs().max())         # a few roundings of 2^-9 each
+        assert float((a - b).abs().max()) > 0                                    # ... and they do round
