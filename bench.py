@@ -1,6 +1,6 @@
 """Headline benchmark: Mixtral-shape bf16 MoE MLP forward+backward on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c1] [--no-cpu]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c1] [--no-cpu] [--compile]
 
 One step = routing prep + GLUMLP forward + backward (dX, d gates, dW1, dW2) on synthetic inputs that
 are resident in HBM before the timed region.  Prints ONE JSON line.  The CPU figure next to it is the
@@ -24,7 +24,7 @@ PEAK_HBM_GBS = 8000.0
 
 def measured_traffic(workload, source_hash):
     """HBM-side bytes per launch of the dominant kernel, from profiles/<workload>_traffic.json - the record a
-    rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE session of this benchmark leaves (profiles/README.md has the commands).
+    rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE session of this benchmark leaves (the record itself names the commands).
     The record names the kernel sources it was measured on; for any other sources the figure would be a guess,
     so None is returned."""
     path = os.path.join(ROOT, "profiles", "%s_traffic.json" % workload)
@@ -98,6 +98,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c2")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--compile", action="store_true",
+                    help="run the module through torch.compile(fullgraph=True): every launch is a registered operator, "
+                         "so the compiled step issues the same kernels as the eager one")
     ap.add_argument("--cpu-tokens", type=int, default=0, help="token count of the CPU sample (default T/3)")
     ap.add_argument("--decode", type=int, default=0, metavar="T",
                     help="forward-only latency of one layer at T tokens (decode regime of the workload's expert "
@@ -270,11 +273,19 @@ def decode_line(args, cfg, torch):
                          hit, 3 if cfg.glu else 2)}}))
 
 
-def mfma_sustained(torch, lib):
+def mfma_sustained(torch):
     """What the matrix pipe sustains on its own (no memory traffic), for all-zero operands and for operands with
     random signs and mantissas: the shader clock follows the operand bits, so the nominal peak that `roofline.frac`
-    is priced against is not reachable on data that is not trivial."""
+    is priced against is not reachable on data that is not trivial.  The kernel lives in a small library of its own
+    (scattermoe_amd/csrc/bench/mfma_probe.hip), not in the product library."""
     import ctypes
+    from scattermoe_amd import _build
+    if not os.path.exists(_build.PROBE_LIB_PATH):
+        return None
+    lib = ctypes.CDLL(_build.PROBE_LIB_PATH)
+    lib.smoe_bench_mfma_rate.restype = ctypes.c_int
+    lib.smoe_bench_mfma_rate.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double),
+                                         ctypes.c_void_p]
     out = torch.empty(65536, dtype=torch.float32, device="cuda:0")
     flop = ctypes.c_double(0.0)
     st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
@@ -283,10 +294,10 @@ def mfma_sustained(torch, lib):
         for iters in (2000, 16000):                  # a short launch to settle the clock, then about 15 ms
             a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             a.record()
-            rc = lib.smoe_mfma_rate_probe(ctypes.c_void_p(out.data_ptr()), iters, kind, ctypes.byref(flop), st)
+            rc = lib.smoe_bench_mfma_rate(out.data_ptr(), iters, kind, ctypes.byref(flop), st)
             b.record()
             torch.cuda.synchronize()
-            assert rc == 0, "smoe_mfma_rate_probe failed: %d" % rc
+            assert rc == 0, "smoe_bench_mfma_rate failed: %d" % rc
         res[name + "_tflops"] = round(flop.value / a.elapsed_time(b) / 1e9, 1)
     res["kernel"] = "independent 32x32x16 bf16 MFMAs, one wave per SIMD on every CU, operands in registers"
     return res
@@ -338,10 +349,12 @@ def main():
     timed = TimedBackend(ops._backend, torch, cfg)
     ops._backend = timed
 
+    fwd = torch.compile(lambda x, p, e: m(x, p, e), fullgraph=True) if args.compile else m
+
     def step():
         for t in leaves:
             t.grad = None
-        y = m(x, p, experts)
+        y = fwd(x, p, experts)
         y.backward(dy)
 
     for _ in range(args.warmup):
@@ -375,7 +388,7 @@ def main():
     k_fl = sum(fl for _, fl in sel) / len(sel)
     achieved = k_fl / (k_ms * 1e-3) / 1e12
     traffic, traffic_src = measured_traffic(cfg.name, _C.source_hash())
-    sustained = mfma_sustained(torch, _C.load())
+    sustained = mfma_sustained(torch)
     roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": traffic, "traffic_source": traffic_src,
                 "kernel": "s2s_mfma_kernel (scatter2scatter products with K-contiguous weights; a product of a few "
@@ -399,6 +412,7 @@ def main():
         "inputs": "router logits, X, dY: CPU generator seed 0 (tests/_inputs.make_inputs order); weights: device "
                   "generator seed 1, N(0, 0.02) (tests/_inputs.make_module)",
         "library_sources": _C.source_hash(),
+        "torch_compile": bool(args.compile),
     }
     if not args.no_cpu:
         tokens = args.cpu_tokens or max(64, cfg.T // 3)            # c2: about 12 s on 16 cores

@@ -333,20 +333,17 @@ int smoe_decode_glu_mlp(const void* X, int64_t sxm, const int64_t* experts, int6
  * Hugging Face blocks the reference patches).  logits (T,E) strides slt,sle, dtype `dtype`; weights_out (T,k)
  * float32 strides swt,swk, selected in descending order of probability; idx_out (T,k) int64 strides sit,sik.
  * Among equal probabilities the lowest expert id is selected first.  E <= 512, k <= 64.
+ * NOT-A-NUMBER LOGITS, a deliberate divergence from the torch composition: torch.softmax turns a row with one NaN
+ * into all NaN and torch.topk ranks NaN above every number, so the reference hands NaN weights (and whatever ids
+ * topk picks) to the expert kernels, where out-of-range or repeated ids are undefined behaviour.  Here a NaN logit
+ * counts as -inf (its expert gets probability 0 and is picked last), and a row that is all NaN / all -inf gets the
+ * uniform distribution: ids are always valid and distinct, weights always finite.  A caller that wants to see a
+ * blown-up router must test the logits itself (torch.isfinite) - this entry point does not report it.
  */
 int smoe_topk_softmax(const void* logits, int64_t slt, int64_t sle, int64_t T, int E, int k, int renormalize,
                       float* weights_out, int64_t swt, int64_t swk, int64_t* idx_out, int64_t sit, int64_t sik,
                       int dtype, void* stream);
 
-/*
- * Measurement aid, no counterpart in the reference and no part of the MoE path: launches a kernel of nothing but
- * independent 32x32x16 bf16 MFMAs (one wave per SIMD on every CU, operands in registers, no memory traffic) and
- * stores the flop count of the launch in *flop_out.  `random_operands` = 0: all-zero operands; 1: random signs and
- * mantissas.  The time of the launch (events on `stream`) gives the rate the matrix pipe sustains at the shader
- * clock the power management grants for such operands; bench.py reports it beside the roofline fraction, which is
- * priced against the nominal peak.  `out`: 65536 floats of device memory (overwritten).
- */
-int smoe_mfma_rate_probe(float* out, int iters, int random_operands, double* flop_out, void* stream);
 
 #ifdef __cplusplus
 }

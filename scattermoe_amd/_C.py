@@ -62,7 +62,6 @@ _SIGNATURES = {
                                    _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _p, _i64, _i64, _int, _i64, _i64,
                                    _int, _int, _int, _p]),
     "smoe_topk_softmax": (_int, [_p, _i64, _i64, _i64, _int, _int, _int, _p, _i64, _i64, _p, _i64, _i64, _int, _p]),
-    "smoe_mfma_rate_probe": (_int, [_p, _int, _int, ctypes.POINTER(ctypes.c_double), _p]),
 }
 
 ERR_UNSUPPORTED = -6

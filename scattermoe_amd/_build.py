@@ -12,8 +12,11 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 OBJ_DIR = os.path.join(CSRC, "build")
 LIB_PATH = os.path.join(PKG_DIR, "libscattermoe_amd.so")
+# measurement aid of bench.py (csrc/bench/): a library of its own, so that the product library holds the MoE path only
+PROBE_SRC = os.path.join(CSRC, "bench", "mfma_probe.hip")
+PROBE_LIB_PATH = os.path.join(PKG_DIR, "libsmoe_bench_probe.so")
 
-SOURCES = ["capi.hip", "route.hip", "group.hip", "s2s_generic.hip", "xty_generic.hip", "gemm_mfma.hip", "fused.hip", "router.hip", "s2s_rowdot.hip", "gemm_f32.hip", "mfma_probe.hip"]
+SOURCES = ["capi.hip", "route.hip", "group.hip", "s2s_generic.hip", "xty_generic.hip", "gemm_mfma.hip", "fused.hip", "router.hip", "s2s_rowdot.hip", "gemm_f32.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
@@ -74,6 +77,10 @@ def build(verbose=False, jobs=None):
     tmp = LIB_PATH + ".tmp"
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp] + objs)
     os.replace(tmp, LIB_PATH)
+    if os.path.exists(PROBE_SRC):
+        tmp = PROBE_LIB_PATH + ".tmp"
+        _run([hipcc] + HIPCC_FLAGS + ["-shared", "-o", tmp, PROBE_SRC])
+        os.replace(tmp, PROBE_LIB_PATH)
     return LIB_PATH
 
 

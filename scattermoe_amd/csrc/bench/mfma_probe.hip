@@ -1,12 +1,12 @@
-// Measurement aid, not part of the MoE path: what the matrix pipe of this GPU sustains on its own.  One wave per
+// Measurement aid of bench.py, built into a library of its own (libsmoe_bench_probe.so): not part of the MoE path,
+// not in the product library or its header.  What the matrix pipe of this GPU sustains on its own.  One wave per
 // SIMD on every CU issues independent 32x32x16 bf16 MFMAs on operands that stay in registers - no memory traffic,
 // no LDS - so the rate is the shader clock the power management grants, and that clock depends on the operand bits
 // (all-zero operands run near the nominal clock, operands with random signs and mantissas 15-25 % below it).
 // bench.py reports both rates beside the roofline fraction, which is priced against the nominal peak.
 #include <hip/hip_runtime.h>
-#include "common.hpp"
 
-namespace smoe {
+namespace {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 probe_bf16x8;
 typedef __attribute__((ext_vector_type(16))) float probe_f32x16;
@@ -48,10 +48,15 @@ __global__ __launch_bounds__(PROBE_THREADS) void mfma_rate_kernel(float* out, in
   out[t] = s;
 }
 
-int launch_mfma_rate_probe(float* out, int iters, int random_operands, double* flop, hipStream_t st) {
-  if (flop) *flop = (double)PROBE_WGS * (PROBE_THREADS / 64) * (double)iters * PROBE_MFMAS * (2.0 * 32 * 32 * 16);
-  hipLaunchKernelGGL(mfma_rate_kernel, dim3(PROBE_WGS), dim3(PROBE_THREADS), 0, st, out, iters, random_operands);
-  return launch_status("mfma_rate_kernel");
-}
+}  // namespace
 
-}  // namespace smoe
+// out: 65536 floats of device memory (overwritten); *flop_out: flop count of the launch.  0 = launched,
+// -1 = NULL pointer, -5 = iters out of range, > 0 = hipError_t of the launch.
+extern "C" int smoe_bench_mfma_rate(float* out, int iters, int random_operands, double* flop_out, void* stream) {
+  if (!out) return -1;
+  if (iters < 1 || iters > (1 << 22)) return -5;
+  if (flop_out) *flop_out = (double)PROBE_WGS * (PROBE_THREADS / 64) * (double)iters * PROBE_MFMAS * (2.0 * 32 * 32 * 16);
+  hipLaunchKernelGGL(mfma_rate_kernel, dim3(PROBE_WGS), dim3(PROBE_THREADS), 0, (hipStream_t)stream, out, iters,
+                     random_operands != 0);
+  return (int)hipGetLastError();
+}

@@ -39,13 +39,6 @@ const char* smoe_last_error(void) { return g_err; }
 #endif
 const char* smoe_source_hash(void) { return SMOE_SOURCE_HASH; }
 
-int smoe_mfma_rate_probe(float* out, int iters, int random_operands, double* flop_out, void* stream) {
-  g_err[0] = 0;
-  if (!out) { set_error("smoe_mfma_rate_probe: NULL pointer"); return SMOE_ERR_NULL; }
-  if (iters < 1 || iters > (1 << 22)) { set_error("smoe_mfma_rate_probe: iters=%d out of range", iters); return SMOE_ERR_RANGE; }
-  return launch_mfma_rate_probe(out, iters, random_operands != 0, flop_out, (hipStream_t)stream);
-}
-
 size_t smoe_route_workspace_bytes(int64_t L, int E) {
   if (L < 0 || E <= 0) return 0;
   return route_workspace_bytes(L, E);

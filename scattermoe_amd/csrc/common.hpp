@@ -279,6 +279,5 @@ int launch_invert_index(const int64_t* idx, int64_t L, int* inv, hipStream_t st)
 int launch_gate_grad_group(const void* Y, int64_t sy, const void* D, int64_t sd, const void* G, int64_t sgt, int64_t sgk,
                            const int64_t* idx, int* inv, void* DY, int64_t sdy, void* DG, int64_t sdgt, int64_t sdgk,
                            int64_t Tn, int k, int N, int dtype, hipStream_t st);
-int launch_mfma_rate_probe(float* out, int iters, int random_operands, double* flop, hipStream_t st);
 
 }  // namespace smoe

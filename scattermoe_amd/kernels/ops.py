@@ -387,6 +387,25 @@ def _s2s_glu_op(X: torch.Tensor, W: torch.Tensor, b: Optional[torch.Tensor], pre
         _backend.glu_fwd(tmp, h, act)
 
 
+@torch.library.custom_op("scattermoe::scatter2scatter_oss_glu", mutates_args={"pre", "h"})
+def _s2s_oss_glu_op(X: torch.Tensor, W: torch.Tensor, b: Optional[torch.Tensor], pre: Optional[torch.Tensor],
+                    h: torch.Tensor, eid: torch.Tensor, idx: torch.Tensor, off: torch.Tensor, k: int,
+                    x_grouped: bool, alpha: float, limit: float) -> None:
+    if not _backend.s2s_oss_glu(X, W, b, pre, h, eid, idx, off, k, x_grouped, alpha, limit):
+        tmp = pre if pre is not None else torch.empty((h.size(0), 2 * h.size(1)), dtype=h.dtype, device=h.device)
+        _backend.s2s(X, W, b, tmp, eid, idx, off, k, x_grouped, True)
+        _backend.oss_glu_fwd(tmp, h, alpha, limit)
+
+
+@torch.library.custom_op("scattermoe::scatter2scatter_oss_glu_bwd", mutates_args={"dpre"})
+def _s2s_oss_glu_bwd_op(DY: torch.Tensor, W: torch.Tensor, pre: torch.Tensor, dpre: torch.Tensor, eid: torch.Tensor,
+                        idx: torch.Tensor, off: torch.Tensor, alpha: float, limit: float) -> None:
+    if not _backend.s2s_oss_glu_bwd(DY, W, pre, dpre, eid, idx, off, alpha, limit):
+        dh = torch.empty((DY.size(0), W.size(2)), dtype=DY.dtype, device=DY.device)
+        _backend.s2s(DY, W, None, dh, eid, idx, off, 1, True, True)
+        _backend.oss_glu_bwd(pre, dh, dpre, alpha, limit)
+
+
 @torch.library.custom_op("scattermoe::scatter2scatter_glu_bwd", mutates_args={"dpre"})
 def _s2s_glu_bwd_op(DY: torch.Tensor, W: torch.Tensor, pre: torch.Tensor, dpre: torch.Tensor, eid: torch.Tensor,
                     idx: torch.Tensor, off: torch.Tensor, act: int) -> None:
@@ -463,8 +482,12 @@ def scatter2scatter(X, W, sorted_expert_idxs, sorted_scattered_idxs, k,
     else:
         assert out.size(0) == L and out.size(1) == N
     if torch.compiler.is_compiling():
-        scatter2scatter_compileable(out, W, X, k, sorted_expert_idxs, sorted_scattered_idxs,
-                                    b, x_grouped, y_grouped)
+        if expert_offsets is None:
+            scatter2scatter_compileable(out, W, X, k, sorted_expert_idxs, sorted_scattered_idxs,
+                                        b, x_grouped, y_grouped)
+        else:       # same launch, without deriving the offsets again from the sorted ids
+            _s2s_offsets_op(out, W, X, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets,
+                            b, x_grouped, y_grouped)
     else:
         _s2s_launch(out, W, X, k, sorted_expert_idxs, sorted_scattered_idxs, b,
                     x_grouped, y_grouped, expert_offsets)
@@ -489,6 +512,16 @@ def scatter2scatter_compileable(
         sorted_expert_idxs: torch.Tensor, sorted_scattered_idxs: torch.Tensor,
         b: Optional[torch.Tensor], x_grouped: bool, y_grouped: bool) -> None:
     _s2s_launch(output, W, X, k, sorted_expert_idxs, sorted_scattered_idxs, b, x_grouped, y_grouped, None)
+
+
+@torch.library.custom_op("scattermoe::scatter2scatter_offsets", mutates_args={"output"})
+def _s2s_offsets_op(
+        output: torch.Tensor, W: torch.Tensor, X: torch.Tensor, k: int,
+        sorted_expert_idxs: torch.Tensor, sorted_scattered_idxs: torch.Tensor, expert_offsets: torch.Tensor,
+        b: Optional[torch.Tensor], x_grouped: bool, y_grouped: bool) -> None:
+    """scattermoe::scatter2scatter for callers that hold the expert offsets (the reference's schema has no such
+    argument: its kernel finds the expert boundaries itself)."""
+    _s2s_launch(output, W, X, k, sorted_expert_idxs, sorted_scattered_idxs, b, x_grouped, y_grouped, expert_offsets)
 
 
 # ------------------------------------------------------------------------------------------------
@@ -516,13 +549,11 @@ def group_bwd_W(DY, X, expert_offsets, E, has_bias=False, like=None, gather=None
     if gather is not None:
         idx, fan_out = gather
         assert idx.size(0) == DY.size(0) and X.size(0) * fan_out == DY.size(0)
-        if (not torch.compiler.is_compiling() and DY.is_cuda and hasattr(_backend, "xty_gathered")
-                and DY.dtype in (torch.bfloat16, torch.float16)):
-            _same_dtype("group_bwd_W", DY, X, DW, Db)
-            if _backend.xty_gathered(DY, X, _as_i64(idx).contiguous(), fan_out, DW, Db,
-                                     _as_i64(expert_offsets).contiguous(), E):
-                return DW, Db
-        X = group(X, idx, fan_out=fan_out, permutation=True)   # `gather` is the routing's index vector
+        if torch.compiler.is_compiling():
+            _xty_gathered_op(E, DW, Db, DY, X, idx, fan_out, expert_offsets)
+        else:
+            _xty_gathered_launch(E, DW, Db, DY, X, idx, fan_out, expert_offsets)
+        return DW, Db
     if torch.compiler.is_compiling():
         groupXtY_compileable(E, DW, Db, DY, X, expert_offsets)
     else:
@@ -535,6 +566,25 @@ def _xty_launch(E, DW, Db, DY, X, expert_offsets):
     assert expert_offsets.numel() == E
     _same_dtype("group_bwd_W", DY, X, DW, Db)
     _backend.xty(DY, X, DW, Db, _as_i64(expert_offsets).contiguous(), E)
+
+
+def _xty_gathered_launch(E, DW, Db, DY, X, idx, fan_out, expert_offsets):
+    """groupXtY over X[idx // fan_out]: one launch that reads the rows of X through idx where the library has one,
+    else the gathered copy and the plain launch."""
+    if DY.is_cuda and hasattr(_backend, "xty_gathered") and DY.dtype in (torch.bfloat16, torch.float16):
+        _same_dtype("group_bwd_W", DY, X, DW, Db)
+        if _backend.xty_gathered(DY, X, _as_i64(idx).contiguous(), fan_out, DW, Db,
+                                 _as_i64(expert_offsets).contiguous(), E):
+            return
+    Xg = torch.empty((idx.size(0), X.size(1)), dtype=X.dtype, device=X.device)
+    _group_launch(X, Xg, None, fan_out, idx, True)            # `idx` is the routing's index vector
+    _xty_launch(E, DW, Db, DY, Xg, expert_offsets)
+
+
+@torch.library.custom_op("scattermoe::groupXtY_gathered", mutates_args={"DW", "Db"})
+def _xty_gathered_op(E: int, DW: torch.Tensor, Db: Optional[torch.Tensor], DY: torch.Tensor, X: torch.Tensor,
+                     idx: torch.Tensor, fan_out: int, expert_offsets: torch.Tensor) -> None:
+    _xty_gathered_launch(E, DW, Db, DY, X, idx, fan_out, expert_offsets)
 
 
 @torch.library.custom_op("scattermoe::groupXtY", mutates_args={"DW", "Db"})
@@ -557,7 +607,10 @@ def group(A, sorted_expert_idxs, coeff=None, fan_out=1, out=None, permutation=Fa
     assert A.size(0) * fan_out == N
     Y = out if out is not None else torch.empty((N, K), dtype=A.dtype, device=A.device)
     if torch.compiler.is_compiling():
-        group_compileable(A, K, N, Y, coeff, coeff is not None, fan_out, sorted_expert_idxs)
+        if permutation:
+            _group_permutation_op(A, K, N, Y, coeff, coeff is not None, fan_out, sorted_expert_idxs)
+        else:
+            group_compileable(A, K, N, Y, coeff, coeff is not None, fan_out, sorted_expert_idxs)
     else:
         _group_launch(A, Y, coeff, fan_out, sorted_expert_idxs, permutation)
         _wrote_into(out)
@@ -582,6 +635,14 @@ def _group_launch(A, Y, coeff, fan_out, idx, permutation=False):
 def group_compileable(A: torch.Tensor, K: int, N: int, Y: torch.Tensor, coeff: Optional[torch.Tensor],
                       has_coeff: bool, fan_out: int, sorted_expert_idxs: torch.Tensor) -> None:
     _group_launch(A, Y, coeff if has_coeff else None, fan_out, sorted_expert_idxs)
+
+
+@torch.library.custom_op("scattermoe::group_permutation", mutates_args={"Y"})
+def _group_permutation_op(A: torch.Tensor, K: int, N: int, Y: torch.Tensor, coeff: Optional[torch.Tensor],
+                          has_coeff: bool, fan_out: int, sorted_expert_idxs: torch.Tensor) -> None:
+    """scattermoe::group for an index vector known to be a permutation (the routing's): same schema, same result,
+    every source row read once."""
+    _group_launch(A, Y, coeff if has_coeff else None, fan_out, sorted_expert_idxs, True)
 
 
 # ------------------------------------------------------------------------------------------------
@@ -720,10 +781,12 @@ def scatter2scatter_glu(X, W, sorted_expert_idxs, sorted_scattered_idxs, k, b=No
         h = torch.empty((L, F), device=X.device, dtype=X.dtype)
         args = (_rows_contiguous(X), W, b, pre, h, _as_i64(sorted_expert_idxs), _as_i64(sorted_scattered_idxs),
                 _as_i64(off), k, x_grouped)
-        if torch.compiler.is_compiling():
-            if not oss:
-                _s2s_glu_op(*args, act)          # falls back to the two launches by itself
-                return pre, h
+        if torch.compiler.is_compiling():       # the operators fall back to the two launches by themselves
+            if oss:
+                _s2s_oss_glu_op(*args, float(alpha), float(limit))
+            else:
+                _s2s_glu_op(*args, act)
+            return pre, h
         elif (_backend.s2s_oss_glu(*args, float(alpha), float(limit)) if oss else _backend.s2s_glu(*args, act)):
             return pre, h
     pre = scatter2scatter(X, W, sorted_expert_idxs, sorted_scattered_idxs, k, b=b, x_grouped=x_grouped,
@@ -750,9 +813,11 @@ def scatter2scatter_glu_bwd(DY, W, pre, sorted_expert_idxs, sorted_scattered_idx
         args = (_rows_contiguous(DY), W, pre_c, dpre, _as_i64(sorted_expert_idxs), _as_i64(sorted_scattered_idxs),
                 _as_i64(off))
         if torch.compiler.is_compiling():
-            if not oss:
+            if oss:
+                _s2s_oss_glu_bwd_op(*args, float(alpha), float(limit))
+            else:
                 _s2s_glu_bwd_op(*args, act)
-                return dpre
+            return dpre
         elif (_backend.s2s_oss_glu_bwd(*args, float(alpha), float(limit)) if oss
               else _backend.s2s_glu_bwd(*args, act)):
             return dpre

@@ -118,6 +118,13 @@ class ParallelLinear(torch.autograd.Function):
 def parallel_linear(inputs, expert_weights, k,
                     sorted_expert_idxs, sorted_scattered_idxs, expert_offsets,
                     expert_biases=None, gates=None, grouped_in=False, grouped_out=False):
+    """Reference parallel_experts.py:136-146, same arguments.
+
+    `sorted_scattered_idxs` must be what `flatten_sort_count` returns for this batch: a permutation of
+    range(tokens * k).  The forward pass already depends on that (with `grouped_out=False` row idx[n] of the output
+    is written by row n: a repeated entry leaves another row unwritten, here as in the reference); the backward pass
+    depends on it too, because the gate-scaled output gradient is written by source row through the inverse
+    permutation - rows of a vector that is no permutation would keep stale contents."""
     return ParallelLinear.apply(inputs, expert_weights, k,
                                 sorted_expert_idxs, sorted_scattered_idxs, expert_offsets,
                                 expert_biases, gates, grouped_in, grouped_out)

@@ -36,7 +36,8 @@ def _experts(T, E, k, seed, skew=False):
 # ---------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("T,E,k", [(1, 8, 2), (3, 1, 1), (256, 8, 2), (512, 8, 4), (2048, 8, 2), (2049, 8, 2),
                                    (8192, 32, 4), (32768, 128, 8), (16384, 8, 2), (5000, 300, 3), (70000, 64, 1),
-                                   (4096, 512, 8), (2000, 700, 5), (16385, 8, 2), (40000, 2000, 1)])
+                                   (4096, 512, 8), (2000, 700, 5), (16385, 8, 2), (40000, 2000, 1),
+                                   (2048, 512, 8)])      # 16384 rows over 512 experts: the most one workgroup sorts
 @pytest.mark.parametrize("dtype", [torch.int64, torch.int32])
 def test_route_bit_exact(T, E, k, dtype):
     experts = _experts(T, E, k, seed=T + E, skew=(E >= 32)).to(dtype)
@@ -331,21 +332,24 @@ def test_slot_sum_bit_exact(T, k, N, dtype):
 
 
 def test_mfma_rate_probe_launches():
-    """The measurement aid behind bench.py's `mfma_sustained`: launches, reports its flop count, and its sums are
-    what the operands say (zeros stay zero; 16-deep products of values below 2 stay finite)."""
+    """The measurement aid behind bench.py's `mfma_sustained` (a library of its own beside the product library):
+    launches, reports its flop count, and its sums are what the operands say (zeros stay zero; 16-deep products of
+    values below 2 stay finite)."""
     import ctypes
-    from scattermoe_amd import _C
-    lib = _C.load()
+    from scattermoe_amd import _build
+    lib = ctypes.CDLL(_build.PROBE_LIB_PATH)
+    fn = lib.smoe_bench_mfma_rate
+    fn.restype = ctypes.c_int
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double), ctypes.c_void_p]
     out = torch.full((65536,), float("nan"), device=DEV)
     flop = ctypes.c_double(0.0)
     st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    assert lib.smoe_mfma_rate_probe(ctypes.c_void_p(out.data_ptr()), 3, 0, ctypes.byref(flop), st) == 0
+    assert fn(out.data_ptr(), 3, 0, ctypes.byref(flop), st) == 0
     torch.cuda.synchronize()
     assert flop.value == 1024 * 3 * 64 * 2.0 * 32 * 32 * 16
     assert bool((out == 0).all())
-    assert lib.smoe_mfma_rate_probe(None, 3, 1, ctypes.byref(flop), st) == -1                 # SMOE_ERR_NULL
-    assert lib.smoe_mfma_rate_probe(ctypes.c_void_p(out.data_ptr()), 0, 1, ctypes.byref(flop), st) == -5   # SMOE_ERR_RANGE
-    assert lib.smoe_mfma_rate_probe(ctypes.c_void_p(out.data_ptr()), 3, 1, ctypes.byref(flop), st) == 0
+    assert fn(None, 3, 1, ctypes.byref(flop), st) == -1
+    assert fn(out.data_ptr(), 0, 1, ctypes.byref(flop), st) == -5
+    assert fn(out.data_ptr(), 3, 1, ctypes.byref(flop), st) == 0
     torch.cuda.synchronize()
     assert bool(torch.isfinite(out).all()) and float(out.abs().max()) > 0
-    assert lib.smoe_last_error() == b""
