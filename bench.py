@@ -391,8 +391,9 @@ def main():
     sustained = mfma_sustained(torch)
     roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": traffic, "traffic_source": traffic_src,
-                "kernel": "s2s_mfma_kernel (scatter2scatter products with K-contiguous weights; a product of a few "
-                          "rounds of tiles plus a remainder runs as two launches and is timed as one)",
+                "kernel": "s2s_mfma_kernel (scatter2scatter products with K-contiguous weights; a product may run as "
+                          "several launches - whole rounds of tiles, remainder, the experts' last tiles in contraction "
+                          "parts and their sum - and is timed as one)",
                 "launches_per_step": len(sel) // args.steps, "avg_launch_ms": round(k_ms, 4),
                 "avg_flop_per_launch": k_fl,
                 "all_s2s_launches_avg_tflops": round(sum(fl for _, fl in allk) / sum(t for t, _ in allk) / 1e9, 1)}

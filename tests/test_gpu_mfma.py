@@ -269,6 +269,38 @@ def test_s2s_last_tiles_with_split_contraction(x_grouped, y_grouped, w_layout, d
     assert torch.equal(via_ops, got)
 
 
+def test_s2s_workspace_that_is_too_small_or_misaligned_is_not_used():
+    """smoe_scatter2scatter_ws with less workspace than it asks for, or with a workspace that is not 16-byte aligned,
+    is exactly smoe_scatter2scatter: same bits, nothing written to the workspace."""
+    from scattermoe_amd import _C
+    lib = _C.load()
+    counts, K, N = SPLIT_COUNTS, 4096, 4096
+    E, L = len(counts), sum(counts)
+    eid, idx, off, g = _routing_with_counts(counts, 1, seed=22)
+    X = torch.randn(L, K, generator=g).bfloat16().to(DEV)
+    W = (torch.randn(E, N, K, generator=g) * 0.03).bfloat16().to(DEV).permute(0, 2, 1)
+    b = torch.randn(E, N, generator=g).bfloat16().to(DEV)
+    eid, idx, off = eid.to(DEV), idx.to(DEV), off.to(DEV)
+    plain = _s2s_through_the_c_abi(X, W, b, eid, idx, off, 1, True, False, workspace=False)
+    need = lib.smoe_scatter2scatter_workspace_bytes(L, K, N, E, _C.float_code(X.dtype))
+    assert need == E * (N // 256) * 4 * 128 * 256 * 4                  # experts x tile columns x parts x one float32 tile
+    ws = torch.full((need + 64,), 0x5a, dtype=torch.uint8, device=DEV)
+    for ptr, size in ((ws.data_ptr(), need - 16), (ws.data_ptr() + 8, need)):
+        Y = torch.full((L, N), float("nan"), dtype=X.dtype, device=DEV)
+        rc = lib.smoe_scatter2scatter_ws(_C.ptr(X), X.stride(0), X.stride(1), _C.ptr(W), W.stride(0), W.stride(1), W.stride(2),
+                                         _C.ptr(b), b.stride(0), b.stride(1), _C.ptr(Y), Y.stride(0), Y.stride(1),
+                                         _C.ptr(eid), _C.ptr(idx), _C.ptr(off), L, K, N, E, 1, 1, 0, _C.float_code(X.dtype),
+                                         ptr, size, _C.stream_ptr(X.device))
+        assert rc == 0, lib.smoe_last_error()
+        torch.cuda.synchronize()
+        assert torch.equal(Y, plain)
+        assert bool((ws == 0x5a).all())
+    # products that would not split ask for none
+    assert lib.smoe_scatter2scatter_workspace_bytes(L, K, 28672, E, _C.float_code(X.dtype)) == 0      # enough tile columns
+    assert lib.smoe_scatter2scatter_workspace_bytes(L, 64, N, E, _C.float_code(X.dtype)) == 0         # short contraction
+    assert lib.smoe_scatter2scatter_workspace_bytes(L, K, N, E, _C.F32) == 0
+
+
 @pytest.mark.parametrize("act", ["SILU", "GPT_OSS"])
 def test_fused_gated_products_with_last_tiles_in_their_own_launch(act):
     """The same row counts through the products that carry the gated unit in their epilogue (forward: saved
