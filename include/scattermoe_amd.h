@@ -127,7 +127,8 @@ int smoe_scatter2scatter(const void* X, int64_t sxm, int64_t sxk,
  * their contraction is cut into parts that run side by side; a second small launch adds the float32 partial
  * sums in a fixed order and writes the rows.  Results are the same on every run, and within float32 rounding
  * of - not bit-identical to - the product without workspace (the additions are grouped differently).
- * workspace == NULL or too small: exactly smoe_scatter2scatter.  The workspace is free again when the launches
+ * workspace == NULL, too small or not 16-byte aligned: exactly smoe_scatter2scatter (the workspace is then not
+ * touched; no error).  The workspace is free again when the launches
  * of the call have run.  smoe_scatter2scatter_workspace_bytes returns 0 for products that would not use one.
  */
 size_t smoe_scatter2scatter_workspace_bytes(int64_t L, int64_t K, int64_t N, int E, int dtype);

@@ -1032,8 +1032,9 @@ __device__ __forceinline__ void epilogue_glu_bwd_staged(const f32x16 (&acc)[TL::
       const int p = (q0 + u) * TL::NT + threadIdx.x;
       const int row = p / CPR, n = n0 + (p % CPR) * 8;
       const T* src = pre + (int64_t)(row0 + (row < rows ? row : 0)) * a.saux + (n < F ? n : 0);
-      p1[decltype(buf)::value][u] = *(const T8*)src;
-      p2[decltype(buf)::value][u] = *(const T8*)(src + F);
+      // read exactly once per step: the non-temporal hint keeps it from displacing operand panels in the L2 (-0.3 %)
+      p1[decltype(buf)::value][u] = __builtin_nontemporal_load((const T8*)src);
+      p2[decltype(buf)::value][u] = __builtin_nontemporal_load((const T8*)(src + F));
     }
   };
   auto work = [&](auto buf, int q0) {
