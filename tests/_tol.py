@@ -7,8 +7,9 @@ Bars (elementwise, `err <= abs + rel * |want|`):
 The absolute term is meant for values of magnitude about one.  Rule used everywhere: when the reference tensor's
 largest magnitude `m` exceeds 1, the absolute term is multiplied by `m` (a sum of n products of 16-bit values
 carries a rounding error that grows with its own magnitude); when `m <= 1` the literal, unscaled bar is asserted.
-`check` also records the observed errors; the session writes them to `gpurun_out/parity_errors.md` (a table of
-max |err|, max |err| / m and the share of the bar that was used) when that folder exists.
+`check` also records the observed errors; at the end of the session they are written, as a table of max |err|,
+max |err| / m and the share of the bar that was used, to the file the environment variable
+SCATTERMOE_PARITY_REPORT names (no report when it is unset).
 """
 import os
 
@@ -78,7 +79,6 @@ def write_report(path):
 
 
 def maybe_write_report():
-    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    out = os.path.join(root, "gpurun_out")
-    if REPORT and os.path.isdir(out):
-        write_report(os.path.join(out, "parity_errors.md"))
+    path = os.environ.get("SCATTERMOE_PARITY_REPORT")
+    if REPORT and path:
+        write_report(path)
