@@ -1,9 +1,9 @@
 """Headline benchmark: Mixtral-shape bf16 MoE MLP forward+backward on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c1] [--no-cpu] [--compile]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c1] [--no-cpu] [--compile] [--forward-only]
 
 One step = routing prep + GLUMLP forward + backward (dX, d gates, dW1, dW2) on synthetic inputs that
-are resident in HBM before the timed region.  Prints ONE JSON line.  The CPU figure next to it is the
+are resident in HBM before the timed region (with --forward-only: routing prep + forward under no_grad).  Prints ONE JSON line.  The CPU figure next to it is the
 naive per-expert PyTorch path (the oracle) timed on the host cores on a reduced token count.
 """
 import argparse
@@ -101,6 +101,9 @@ def parse():
     ap.add_argument("--compile", action="store_true",
                     help="run the module through torch.compile(fullgraph=True): every launch is a registered operator, "
                          "so the compiled step issues the same kernels as the eager one")
+    ap.add_argument("--forward-only", action="store_true",
+                    help="time the forward pass alone under no_grad (inference: the pre-activation is not stored); the "
+                         "metric becomes moe_mlp_fwd_tokens_per_s")
     ap.add_argument("--cpu-tokens", type=int, default=0, help="token count of the CPU sample (default T/3)")
     ap.add_argument("--decode", type=int, default=0, metavar="T",
                     help="forward-only latency of one layer at T tokens (decode regime of the workload's expert "
@@ -163,8 +166,9 @@ class TimedBackend:
                            2.0 * eid.numel() * DY.size(1) * W.size(2), W.stride(1) == 1, "l2_dx")
 
 
-def cpu_baseline(cfg, tokens, torch):
-    """Naive per-expert PyTorch path (oracle), fp32, forward + autograd backward, on `tokens` tokens."""
+def cpu_baseline(cfg, tokens, torch, forward_only=False):
+    """Naive per-expert PyTorch path (oracle), fp32, forward + autograd backward (or the forward alone), on `tokens`
+    tokens."""
     import oracle
     from _inputs import make_inputs, scaled
     small = scaled(cfg, T=tokens)
@@ -182,12 +186,16 @@ def cpu_baseline(cfg, tokens, torch):
     x = t["x"].requires_grad_()
     p = t["p"].requires_grad_()
     t0 = time.perf_counter()
-    y = oracle.naive_expert_forward(x, p, t["experts"], W1, W2, hidden, b1, b2)
-    y.backward(t["dy"])
+    if forward_only:
+        with torch.no_grad():
+            oracle.naive_expert_forward(x, p, t["experts"], W1, W2, hidden, b1, b2)
+    else:
+        y = oracle.naive_expert_forward(x, p, t["experts"], W1, W2, hidden, b1, b2)
+        y.backward(t["dy"])
     dt = time.perf_counter() - t0
     return {"value": tokens / dt, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": "%s at T=%d of %d tokens (same d, f, E, k), fp32, 1 forward+backward, %.1f s; host has %d cpus"
-                      % (cfg.name, tokens, cfg.T, dt, os.cpu_count())}
+            "sample": "%s at T=%d of %d tokens (same d, f, E, k), fp32, 1 %s, %.1f s; host has %d cpus"
+                      % (cfg.name, tokens, cfg.T, "forward" if forward_only else "forward+backward", dt, os.cpu_count())}
 
 
 def profile_one_kernel(args, cfg, torch, ops):
@@ -352,6 +360,10 @@ def main():
     fwd = torch.compile(lambda x, p, e: m(x, p, e), fullgraph=True) if args.compile else m
 
     def step():
+        if args.forward_only:
+            with torch.no_grad():
+                fwd(x, p, experts)
+            return
         for t in leaves:
             t.grad = None
         y = fwd(x, p, experts)
@@ -369,7 +381,9 @@ def main():
     timed.on = False
 
     L = cfg.T * cfg.k
-    flops_step = (18.0 if cfg.glu else 12.0) * L * cfg.d * cfg.f
+    flops_step = (18.0 if cfg.glu else 12.0) * L * cfg.d * cfg.f          # forward + both gradients of both layers
+    if args.forward_only:
+        flops_step /= 3.0
     ms = dt / args.steps * 1e3
     tflops = flops_step / (ms * 1e-3) / 1e12
 
@@ -399,12 +413,12 @@ def main():
                 "all_s2s_launches_avg_tflops": round(sum(fl for _, fl in allk) / sum(t for t, _ in allk) / 1e9, 1)}
 
     out = {
-        "metric": "moe_mlp_fwd_bwd_tokens_per_s", "value": round(cfg.T * args.steps / dt, 1), "unit": "tokens/s",
+        "metric": "moe_mlp_fwd_tokens_per_s" if args.forward_only else "moe_mlp_fwd_bwd_tokens_per_s", "value": round(cfg.T * args.steps / dt, 1), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": {torch.bfloat16: "bf16", torch.float32: "f32", torch.float16: "f16"}[dtype], "data": "synthetic",
-        "config": {"workload": "%s: MoE MLP fwd+bwd T=%d d_model=%d d_ff=%d E=%d top_k=%d %s%s" % (
-            cfg.name, cfg.T, cfg.d, cfg.f, cfg.E, cfg.k, "SwiGLU" if cfg.glu else "GELU", " +bias" if cfg.bias else ""),
+        "config": {"workload": "%s: MoE MLP %s T=%d d_model=%d d_ff=%d E=%d top_k=%d %s%s" % (
+            cfg.name, "forward (inference)" if args.forward_only else "fwd+bwd", cfg.T, cfg.d, cfg.f, cfg.E, cfg.k, "SwiGLU" if cfg.glu else "GELU", " +bias" if cfg.bias else ""),
             "tokens": cfg.T, "rows": L},
         "tflops": round(tflops, 1), "frac_of_bf16_mfma_peak": round(tflops / PEAK_BF16_TFLOPS, 4),
         "roofline": roofline,
@@ -417,7 +431,7 @@ def main():
     }
     if not args.no_cpu:
         tokens = args.cpu_tokens or max(64, cfg.T // 3)            # c2: about 12 s on 16 cores
-        out["cpu_baseline"] = cpu_baseline(cfg, tokens, torch)
+        out["cpu_baseline"] = cpu_baseline(cfg, tokens, torch, args.forward_only)
     print(json.dumps(out))
 
 
